@@ -361,19 +361,29 @@ enum {
                                               channels, the head's output turned back by the query's position;
                                        right  a real-gated linear recurrent unit behind a short causal convolution:
                                               a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u, out = S * gelu_tanh(y) */
-    ZG_LM_MIX_CHANNEL_DELTA = 4     /* gated delta rule with a decay per key channel: S = diag(g) S; u = beta (v - S^T k);
+    ZG_LM_MIX_CHANNEL_DELTA = 4,    /* gated delta rule with a decay per key channel: S = diag(g) S; u = beta (v - S^T k);
                                        S += k u^T; o = S^T q;  q, k, v behind short causal convolutions + silu, q and k of unit
                                        length, the decay and the output gate through two-step (low-rank) projections */
+    ZG_LM_MIX_WINDOW_LINEAR = 5     /* two branches on the same input, c_left * left + c_right * right:
+                                       left   grouped-query softmax attention (no rotation) whose q, k, v = conv(W h + b) pass a short
+                                              causal convolution and whose q and k are RMS-normed over the WHOLE projection; a query sees
+                                              the keys inside its window and, beyond it, the first keep_first tokens of the sequence;
+                                              the heads are gated by sigmoid(W_g h), the output projection has a bias;
+                                       right  linear attention with one fixed decay per head: q, k, v = silu(W h), S = decay_h S + k v^T,
+                                              o = S^T q; the heads RMS-normed together, gated by sigmoid(W_g h) */
 };
 enum { ZG_LM_FF_NONE = 0, ZG_LM_FF_DENSE = 1 /* down(relu(up h)^2) */, ZG_LM_FF_MOE = 2 /* top-k of `experts` units */ };
 /* Activation of an expert (ff_act) and the rule of the router (router) of ZG_LM_FF_MOE. */
 enum {
     ZG_LM_ACT_GLU_SILU = 0, /* down(silu(gate h) * up h): tensors e<j>.gate / up / down */
-    ZG_LM_ACT_GELU = 1      /* down(gelu(up h)), the exact (erf) form: tensors e<j>.up / down */
+    ZG_LM_ACT_GELU = 1,     /* down(gelu(up h)), the exact (erf) form: tensors e<j>.up / down */
+    ZG_LM_ACT_GLU_CLIPPED = 2 /* down(g sigmoid(1.702 g) (u + 1)), g = min(gate h, ff_limit), u = clamp(up h, -ff_limit, ff_limit) */
 };
 enum {
     ZG_LM_ROUTE_SOFTMAX_ALL = 0, /* s = softmax over all experts; the `top` largest s + correction; weights s */
-    ZG_LM_ROUTE_TOP_LOGITS = 1   /* z = router h + bias (`router.b`); the `top` largest z; weights softmax over the chosen z */
+    ZG_LM_ROUTE_TOP_LOGITS = 1,  /* z = router h + bias (`router.b`); the `top` largest z; weights softmax over the chosen z */
+    ZG_LM_ROUTE_SIGMOID_INPUT = 2 /* s = sigmoid(router h); the `top` largest; the weight s (not renormalised) multiplies the expert's
+                                     INPUT: the sublayer's output is the plain sum of expert(s h) */
 };
 enum { ZG_LM_ROT_PLAIN = 0, ZG_LM_ROT_YARN = 1 /* blend by pair index, amplitude factor */, ZG_LM_ROT_BANDS = 2 /* by wavelength: see rot_* */ };
 typedef struct {
@@ -396,12 +406,25 @@ typedef struct {
     int conv;                     /* delta rule: taps of the convolutions on q, k, v */
     int decay_rank, gate_rank;    /* delta rule: inner sizes of the two-step projections of the decay and of the output gate */
     int ff_act, router;           /* ZG_LM_ACT_*, ZG_LM_ROUTE_* */
+    int keep_first;               /* windowed attention: the first keep_first tokens of a sequence stay visible behind the window */
+    float left_scale, right_scale; /* window + linear pair: factors of the two branches in their sum */
+    int lin_heads, lin_dim, lin_vdim; /* window + linear pair: heads, key and value channels per head of the linear-attention branch
+                                         (its decays: the fp32 tensor `mix.right.decay` [lin_heads], which the host fills from config.json) */
+    float ff_limit;               /* ZG_LM_ACT_GLU_CLIPPED: the experts' clip */
+    int shared_width;             /* > 0: a shared expert of this hidden width (same activation) runs for every token and is added,
+                                     times sigmoid(shared.sg . h) (tensors shared.gate / up / down / sg) */
+    float shared_limit;           /* its clip */
 } zg_lm_layer;
 enum {
     ZG_LM_F32 = 1 << 0,     /* true 32-bit products everywhere */
     ZG_LM_NO_GRAPH = 1 << 1, /* launch the kernels of a decode step one by one instead of replaying the hipGraph captured for its batch size */
     ZG_LM_TIED_HEAD = 1 << 2, /* logits = embed . norm(x): there is no `head` tensor */
-    ZG_LM_LOOP_READD = 1 << 3 /* every repetition of the looped span but the first starts by adding the embedding output to x */
+    ZG_LM_LOOP_READD = 1 << 3, /* every repetition of the looped span but the first starts by adding the embedding output to x */
+    ZG_LM_SIDE_BY_SIDE = 1 << 4, /* a layer is x += mixer(norm1(x)) + ff(norm2(x)), both sublayers reading the same x; norm weights are
+                                    plain factors (not offsets from one), no norm behind a sublayer (no norm1b / norm2b), no token
+                                    shift; `final.norm` is a plain factor too */
+    ZG_LM_SINUSOID_POSITIONS = 1 << 5 /* the embedding output gets the position's vector added: entry 2i = sin(p 10000^(-2i/width)),
+                                         entry 2i + 1 = cos of the same angle (fp32 position x fp32 frequency) */
 };
 typedef struct {
     size_t vocab, width, n_layers;
@@ -417,6 +440,8 @@ typedef struct {
     int canon_taps;         /* 0: the sublayer input of the mixer is the token shift (tensor `shift`).  >= 1: BOTH sublayers read
                                h + conv(h), a causal convolution per channel over the last canon_taps tokens (tensors `canon1`,
                                `canon2` [width][taps], last column = the current token); a slot keeps the taps - 1 last inputs */
+    float logit_scale;      /* logits = head . norm(x) * logit_scale (0: 1) */
+    float logit_softcap;    /* > 0: logits <- cap tanh(logits / cap) */
 } zg_lm_config;
 typedef struct zg_lm zg_lm;
 /* One arena for weights, state and scratch; the handle owns a stream on `device`.  Needs no zg_init. */
@@ -425,8 +450,11 @@ int zg_lm_destroy(zg_lm* g);
 /* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift|canon1|canon2`,
  * `l<i>.mix.*` (hgrn2: q f f.b lower v norm o; latent attention: dq dq.norm uq dkv dkv.norm uk uv o; parallel: left.q left.k
  * left.v left.sink left.talk left.o left.out right.y right.y.b right.x right.x.b right.conv right.conv.b right.ra right.ra.b
- * right.ri right.ri.b right.lam right.o right.out; delta rule: q q.conv k k.conv v v.conv b A_log dt_bias a1 a2 g1 g2 norm o)
- * and `l<i>.mlp.*` (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router, and correction or router.b).  data: fp32 on the host, `len` elements, matrices
+ * right.ri right.ri.b right.lam right.o right.out; delta rule: q q.conv k k.conv v v.conv b A_log dt_bias a1 a2 g1 g2 norm o;
+ * window + linear pair: left.q|k|v with .b and .conv each, left.q.norm left.k.norm left.g left.o left.o.b right.q right.k right.v
+ * right.g right.norm right.o right.decay)
+ * and `l<i>.mlp.*` (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router, and correction or router.b; shared.gate shared.up
+ * shared.down shared.sg).  data: fp32 on the host, `len` elements, matrices
  * [out][in] row-major; matrices are stored bf16 (round to nearest even).  ZG_ERR_ARG for a name the configuration does not have. */
 int zg_lm_load_tensor(zg_lm* g, const char* name, const float* data, size_t len);
 /* How many tensors of the configuration have not been loaded; names_out (may be NULL) receives them, space separated. */

@@ -49,7 +49,9 @@ class LmLayer(C.Structure):
                 ("rot_factor", C.c_float), ("rot_original", C.c_float), ("rot_fast", C.c_float), ("rot_slow", C.c_float), ("ff", C.c_int),
                 ("ff_width", C.c_int), ("experts", C.c_int), ("top", C.c_int), ("kv_heads", C.c_int), ("window", C.c_int), ("lru_width", C.c_int),
                 ("lru_blocks", C.c_int), ("lru_conv", C.c_int), ("conv", C.c_int), ("decay_rank", C.c_int), ("gate_rank", C.c_int),
-                ("ff_act", C.c_int), ("router", C.c_int)]
+                ("ff_act", C.c_int), ("router", C.c_int), ("keep_first", C.c_int), ("left_scale", C.c_float), ("right_scale", C.c_float),
+                ("lin_heads", C.c_int), ("lin_dim", C.c_int), ("lin_vdim", C.c_int), ("ff_limit", C.c_float), ("shared_width", C.c_int),
+                ("shared_limit", C.c_float)]
 
 
 class LmConfig(C.Structure):
@@ -57,7 +59,8 @@ class LmConfig(C.Structure):
 
     _fields_ = [("vocab", sz), ("width", sz), ("n_layers", sz), ("layers", C.POINTER(LmLayer)), ("loop_start", C.c_int), ("loop_stop", C.c_int),
                 ("loop_times", C.c_int), ("norm_eps", C.c_float), ("max_tokens", sz), ("max_seqs", sz), ("max_step_tokens", sz),
-                ("page_tokens", sz), ("flags", C.c_uint), ("embed_scale", C.c_float), ("canon_taps", C.c_int)]
+                ("page_tokens", sz), ("flags", C.c_uint), ("embed_scale", C.c_float), ("canon_taps", C.c_int), ("logit_scale", C.c_float),
+                ("logit_softcap", C.c_float)]
 
 
 class LmEntry(C.Structure):
@@ -66,12 +69,12 @@ class LmEntry(C.Structure):
     _fields_ = [("seq", C.c_int), ("tokens", vp), ("n_tokens", sz), ("want", vp), ("n_want", sz)]
 
 
-LM_MIX_HGRN2, LM_MIX_LATENT_ATTENTION, LM_MIX_PARALLEL, LM_MIX_CHANNEL_DELTA = 1, 2, 3, 4
+LM_MIX_HGRN2, LM_MIX_LATENT_ATTENTION, LM_MIX_PARALLEL, LM_MIX_CHANNEL_DELTA, LM_MIX_WINDOW_LINEAR = 1, 2, 3, 4, 5
 LM_FF_NONE, LM_FF_DENSE, LM_FF_MOE = 0, 1, 2
-LM_ACT_GLU_SILU, LM_ACT_GELU = 0, 1
-LM_ROUTE_SOFTMAX_ALL, LM_ROUTE_TOP_LOGITS = 0, 1
+LM_ACT_GLU_SILU, LM_ACT_GELU, LM_ACT_GLU_CLIPPED = 0, 1, 2
+LM_ROUTE_SOFTMAX_ALL, LM_ROUTE_TOP_LOGITS, LM_ROUTE_SIGMOID_INPUT = 0, 1, 2
 LM_ROT_PLAIN, LM_ROT_YARN, LM_ROT_BANDS = 0, 1, 2
-LM_F32, LM_NO_GRAPH, LM_TIED_HEAD, LM_LOOP_READD = 1, 2, 4, 8
+LM_F32, LM_NO_GRAPH, LM_TIED_HEAD, LM_LOOP_READD, LM_SIDE_BY_SIDE, LM_SINUSOID_POSITIONS = 1, 2, 4, 8, 16, 32
 
 # the layered-model tier (present in both libraries)
 LM_SIGNATURES = {

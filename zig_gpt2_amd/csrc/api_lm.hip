@@ -17,6 +17,12 @@
 // attention caches rotated keys and rotated values per token in the paged cache, through the same page table as the latents;
 // pages that every attention pass's window has left behind return to the pool while the sequence is still open.
 //
+// Designs whose two sublayers stand side by side (x += mixer(norm1(x)) + ff(norm2(x))) leave a layer's sums open: the next
+// layer's norm kernel adds them to x on its way (one statistic serves both norms), the last layer's are added in front of the
+// final norm.  Their window + linear-attention mixer keeps, per slot and layer, the tail of the q / k / v convolutions and the
+// [heads][dim][vdim] state of the linear attention in the same block of sequence state; its keys (normed) and values go to the
+// paged cache as the other windowed attention's do.
+//
 // Latent attention runs in its absorbed form in prompts and in decoding alike: score_j = (W_uk^T q_nope) . c_j + q_rot . k_rot_j,
 // out = W_uv (sum_j p_j c_j) — only the latent c_j and the rotated key part are cached, and a portion of a prompt needs nothing
 // of the tokens before it but their cache rows.
@@ -44,6 +50,7 @@ struct Tensor {
     void* dev = nullptr;
     bool matrix = false;  // bf16 storage
     size_t rows = 0, cols = 0;
+    size_t ld = 0;            // > 0: the rows lie ld elements apart (a column block of a wider matrix)
     int transpose_heads = 0;  // > 0: source [heads * d][cols] is stored as [heads][cols][d]
     int init = INIT_MATRIX;
     bool loaded = false;
@@ -71,6 +78,10 @@ struct LayerW {
     // delta rule
     bf16_t *a2 = nullptr, *g2 = nullptr;
     float *a_log = nullptr, *dt_bias = nullptr;
+    // window + linear pair: output projections of both branches side by side in one matrix ([W][H V + HR VR]), biases of q | k | v
+    // in one vector, the whole-projection norms, the shared expert ([gate | up | gate logit] rows)
+    bf16_t *ocat = nullptr, *sgu = nullptr, *sdown = nullptr;
+    float *qkv_bias = nullptr, *qnorm = nullptr, *knorm = nullptr, *rnorm = nullptr, *obias = nullptr, *decay = nullptr;
 };
 
 struct Pass {
@@ -117,8 +128,8 @@ struct Sampler {
     int32_t* tokens_out;  // host, indexed by output row
 };
 
-__global__ __launch_bounds__(256) void fill_kernel(void* dst, size_t n, uint64_t key, int kind, float std_) {
-    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+__global__ __launch_bounds__(256) void fill_kernel(void* dst, size_t n, uint64_t key, int kind, float std_, size_t cols, size_t ld) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     uint64_t z = key + (i + 1) * 0x9E3779B97F4A7C15ULL;
     z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ULL;
@@ -126,6 +137,7 @@ __global__ __launch_bounds__(256) void fill_kernel(void* dst, size_t n, uint64_t
     z ^= z >> 31;
     const float s4 = (float)((int)((z & 0xFFFF) + ((z >> 16) & 0xFFFF) + ((z >> 32) & 0xFFFF) + (z >> 48)) - 131070) * (1.0f / 37837.227f);
     const float u = (float)(uint32_t)(z >> 40) * 5.9604644775390625e-08f;
+    i = (i / cols) * ld + i % cols;
     if (kind == INIT_MATRIX) reinterpret_cast<bf16_t*>(dst)[i] = f32_to_bf16_rne(s4 * std_);
     else if (kind == INIT_OFFSET) reinterpret_cast<float*>(dst)[i] = s4 * 0.05f;
     else if (kind == INIT_UNIT) reinterpret_cast<float*>(dst)[i] = u;
@@ -135,6 +147,11 @@ __global__ __launch_bounds__(256) void fill_kernel(void* dst, size_t n, uint64_t
 __global__ __launch_bounds__(256) void zero_kernel(float* p, size_t n) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) p[i] = 0.0f;
+}
+
+__global__ __launch_bounds__(256) void ones_kernel(float* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 1.0f;
 }
 
 }  // namespace
@@ -166,8 +183,12 @@ struct zg_lm {
     float* seq_state = nullptr;  // [NS][seq_floats]: convolution tails and recurrent states of the passes that have them
     size_t seq_floats = 0;
     int canon = 0;        // taps of the sublayers' input convolution (0: token shift)
-    int keep_tokens = 0;  // > 0: no attention pass looks further back than this many tokens
+    int keep_tokens = 0;  // > 0: no attention pass looks further back than this many tokens ...
+    int keep_first = 0;   // ... except at the first keep_first tokens of the sequence, which some pass keeps in sight
+    int keep_pages = 0;   // pages that hold those first tokens: never returned while the sequence is open
     float embed_scale = 1.0f;
+    bool side = false;          // ZG_LM_SIDE_BY_SIDE
+    float* pos_freq = nullptr;  // ZG_LM_SINUSOID_POSITIONS: frequency of every pair of channels
     int* page_table = nullptr;  // [NS][max_pages]
     std::vector<Slot> slots;
     std::vector<int> free_pages;
@@ -215,6 +236,17 @@ void layout(zg_lm* g, Bump& b) {
         t.init = INIT_MATRIX;
         T[name] = t;
     };
+    // columns [col0, col0 + cols) of a matrix whose rows are ld wide
+    auto mat_cols = [&](const std::string& name, bf16_t* base, size_t rows, size_t ld, size_t col0, size_t cols) {
+        Tensor t;
+        t.dev = base ? base + col0 : nullptr;
+        t.matrix = true;
+        t.rows = rows;
+        t.cols = cols;
+        t.ld = ld;
+        t.init = INIT_MATRIX;
+        T[name] = t;
+    };
     auto vec = [&](const std::string& name, float*& p, size_t n, int init) {
         p = b.take<float>(n);
         Tensor t;
@@ -241,17 +273,21 @@ void layout(zg_lm* g, Bump& b) {
         g->head = b.take<bf16_t>(V * W);
         mat("head", g->head, 0, V, W);
     }
-    vec("final.norm", g->final_norm, W, INIT_OFFSET);
+    vec("final.norm", g->final_norm, W, g->side ? INIT_PLAIN : INIT_OFFSET);
+    if (g->cfg.flags & ZG_LM_SINUSOID_POSITIONS) g->pos_freq = b.take<float>((W + 1) / 2);
     size_t max_t = 1, max_win = 0, max_win_few = 0;
     size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
     for (size_t i = 0; i < g->layers.size(); ++i) {
         LayerW& L = g->layers[i];
         const zg_lm_layer& d = L.d;
         const std::string p = "l" + std::to_string(i) + ".";
-        vec(p + "norm1", L.norm1, W, INIT_OFFSET);
-        vec(p + "norm1b", L.norm1b, W, INIT_OFFSET);
-        if (taps == 0) vec(p + "shift", L.shift, W, INIT_UNIT);
-        else vec(p + "canon1", L.canon1, W * taps, INIT_OFFSET);
+        vec(p + "norm1", L.norm1, W, g->side ? INIT_PLAIN : INIT_OFFSET);
+        if (g->side) {
+        } else {
+            vec(p + "norm1b", L.norm1b, W, INIT_OFFSET);
+            if (taps == 0) vec(p + "shift", L.shift, W, INIT_UNIT);
+            else vec(p + "canon1", L.canon1, W * taps, INIT_OFFSET);
+        }
         const size_t H = d.heads, D = d.dim, Vd = d.vdim;
         if (d.mixer == ZG_LM_MIX_PARALLEL) {
             const size_t G = d.kv_heads, C = d.lru_width, NB = d.lru_blocks, BS = C / NB, HV = H * Vd;
@@ -288,6 +324,46 @@ void layout(zg_lm* g, Bump& b) {
             max_o = std::max(max_o, HV);
             max_t = std::max(max_t, C);
             const int cap = d.window > 0 ? d.window : g->max_pages * g->P;
+            max_win = std::max(max_win, window_split_workspace((int)MS, (int)H, (int)Vd, cap, nullptr));
+            max_win_few = std::max(max_win_few, window_split_workspace(kGemvMaxRows, (int)H, (int)Vd, cap, nullptr));
+        } else if (d.mixer == ZG_LM_MIX_WINDOW_LINEAR) {
+            const size_t G = d.kv_heads, HD = H * D, GD = G * D, GV = G * Vd, CC = HD + GD + GV, HV = H * Vd;
+            const size_t HR = d.lin_heads, HRD = HR * d.lin_dim, HRV = HR * d.lin_vdim, NP = CC + HV + 2 * HRD + 2 * HRV;
+            const size_t ct = std::max(1, d.conv);
+            L.n_cat = (int)NP;
+            L.wcat = b.take<bf16_t>(NP * W);  // left q | k | v | gate, right q | k | v | gate
+            const std::string l = p + "mix.left.", r = p + "mix.right.";
+            mat(l + "q", L.wcat, 0, HD, W);
+            mat(l + "k", L.wcat, HD, GD, W);
+            mat(l + "v", L.wcat, HD + GD, GV, W);
+            mat(l + "g", L.wcat, CC, HV, W);
+            mat(r + "q", L.wcat, CC + HV, HRD, W);
+            mat(r + "k", L.wcat, CC + HV + HRD, HRD, W);
+            mat(r + "v", L.wcat, CC + HV + 2 * HRD, HRV, W);
+            mat(r + "g", L.wcat, CC + HV + 2 * HRD + HRV, HRV, W);
+            L.qkv_bias = b.take<float>(CC);
+            vec_at(l + "q.b", L.qkv_bias, 0, HD, INIT_OFFSET);
+            vec_at(l + "k.b", L.qkv_bias, HD, GD, INIT_OFFSET);
+            vec_at(l + "v.b", L.qkv_bias, HD + GD, GV, INIT_OFFSET);
+            L.convw = b.take<float>(CC * ct);  // without a convolution: one tap of weight one, set at creation
+            if (d.conv >= 1) {
+                vec_at(l + "q.conv", L.convw, 0, HD * ct, INIT_OFFSET);
+                vec_at(l + "k.conv", L.convw, HD * ct, GD * ct, INIT_OFFSET);
+                vec_at(l + "v.conv", L.convw, (HD + GD) * ct, GV * ct, INIT_OFFSET);
+            }
+            vec(l + "q.norm", L.qnorm, HD, INIT_PLAIN);
+            vec(l + "k.norm", L.knorm, GD, INIT_PLAIN);
+            L.ocat = b.take<bf16_t>(W * (HV + HRV));
+            mat_cols(l + "o", L.ocat, W, HV + HRV, 0, HV);
+            mat_cols(r + "o", L.ocat, W, HV + HRV, HV, HRV);
+            vec(l + "o.b", L.obias, W, INIT_OFFSET);
+            vec(r + "norm", L.rnorm, HRV, INIT_PLAIN);
+            vec(r + "decay", L.decay, HR, INIT_UNIT);
+            max_proj = std::max(max_proj, NP);
+            max_o = std::max(max_o, HV + HRV);
+            max_t = std::max(max_t, std::max(CC, W));
+            max_scan = std::max(max_scan, HRD * d.lin_vdim + HRD);
+            const int cap = d.window > 0 ? d.window + d.keep_first : g->max_pages * g->P;
             max_win = std::max(max_win, window_split_workspace((int)MS, (int)H, (int)Vd, cap, nullptr));
             max_win_few = std::max(max_win_few, window_split_workspace(kGemvMaxRows, (int)H, (int)Vd, cap, nullptr));
         } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
@@ -355,9 +431,9 @@ void layout(zg_lm* g, Bump& b) {
             max_o = std::max(max_o, HV);
         }
         if (d.ff != ZG_LM_FF_NONE) {
-            vec(p + "norm2", L.norm2, W, INIT_OFFSET);
-            vec(p + "norm2b", L.norm2b, W, INIT_OFFSET);
-            if (taps) vec(p + "canon2", L.canon2, W * taps, INIT_OFFSET);
+            vec(p + "norm2", L.norm2, W, g->side ? INIT_PLAIN : INIT_OFFSET);
+            if (!g->side) vec(p + "norm2b", L.norm2b, W, INIT_OFFSET);
+            if (taps && !g->side) vec(p + "canon2", L.canon2, W * taps, INIT_OFFSET);
         }
         const size_t F = d.ff_width;
         if (d.ff == ZG_LM_FF_DENSE) {
@@ -367,7 +443,7 @@ void layout(zg_lm* g, Bump& b) {
             mat(p + "mlp.down", L.down, 0, W, F);
             max_ff = std::max(max_ff, F);
         } else if (d.ff == ZG_LM_FF_MOE) {
-            const size_t E = d.experts, UF = d.ff_act == ZG_LM_ACT_GLU_SILU ? 2 * F : F;  // rows of an expert's first matrix
+            const size_t E = d.experts, UF = d.ff_act == ZG_LM_ACT_GELU ? F : 2 * F;  // rows of an expert's first matrix
             L.gu = b.take<bf16_t>(E * UF * W);
             L.edown = b.take<bf16_t>(E * W * F);
             for (size_t e = 0; e < E; ++e) {
@@ -378,7 +454,18 @@ void layout(zg_lm* g, Bump& b) {
             }
             L.router = b.take<bf16_t>(E * W);
             mat(p + "mlp.router", L.router, 0, E, W);
-            vec(p + (d.router == ZG_LM_ROUTE_TOP_LOGITS ? "mlp.router.b" : "mlp.correction"), L.correction, E, INIT_OFFSET);
+            if (d.router != ZG_LM_ROUTE_SIGMOID_INPUT)
+                vec(p + (d.router == ZG_LM_ROUTE_TOP_LOGITS ? "mlp.router.b" : "mlp.correction"), L.correction, E, INIT_OFFSET);
+            if (d.shared_width > 0) {  // the shared expert: gate | up rows and, behind them, the row of its gate logit
+                const size_t S = d.shared_width;
+                L.sgu = b.take<bf16_t>((2 * S + 1) * W);
+                mat(p + "mlp.shared.gate", L.sgu, 0, S, W);
+                mat(p + "mlp.shared.up", L.sgu, S, S, W);
+                mat(p + "mlp.shared.sg", L.sgu, 2 * S, 1, W);
+                L.sdown = b.take<bf16_t>(W * S);
+                mat(p + "mlp.shared.down", L.sdown, 0, W, S);
+                max_t = std::max(max_t, std::max(2 * S + 1, W));
+            }
             max_assign = std::max(max_assign, (size_t)d.top);
             max_gu = std::max(max_gu, (size_t)d.top * UF);
             max_hb = std::max(max_hb, (size_t)d.top * F);
@@ -418,6 +505,11 @@ void layout(zg_lm* g, Bump& b) {
             sq += (size_t)(d.conv - 1) * (2 * d.kv_heads * d.dim + d.heads * d.vdim);
             ps.rec_off = sq;
             sq += (size_t)d.heads * d.dim * d.vdim;
+        } else if (d.mixer == ZG_LM_MIX_WINDOW_LINEAR) {
+            ps.conv_off = sq;
+            sq += (size_t)(std::max(1, d.conv) - 1) * ((size_t)d.heads * d.dim + (size_t)d.kv_heads * (d.dim + d.vdim));
+            ps.rec_off = sq;
+            sq += (size_t)d.lin_heads * d.lin_dim * d.lin_vdim;
         }
     }
     g->seq_floats = sq;
@@ -426,7 +518,8 @@ void layout(zg_lm* g, Bump& b) {
     for (Pass& ps : g->passes) {
         const zg_lm_layer& d = g->layers[ps.layer].d;
         if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION) ps.cache = b.take<float>((size_t)g->n_pages * g->P * (d.kv_rank + d.rot_dim));
-        if (d.mixer == ZG_LM_MIX_PARALLEL) ps.cache = b.take<float>((size_t)g->n_pages * g->P * d.kv_heads * (d.dim + d.vdim));
+        if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_WINDOW_LINEAR)
+            ps.cache = b.take<float>((size_t)g->n_pages * g->P * d.kv_heads * (d.dim + d.vdim));
     }
     // scratch
     g->x = b.take<float>(MS * W);
@@ -516,10 +609,10 @@ void rotary_table(const zg_lm_layer& d, std::vector<float>& freq, float& amp) {
     }
 }
 
-int check_layer(const zg_lm_layer& d, size_t i) {
-    ZG_REQUIRE(d.mixer >= ZG_LM_MIX_HGRN2 && d.mixer <= ZG_LM_MIX_CHANNEL_DELTA, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
+int check_layer(const zg_lm_layer& d, size_t i, unsigned flags) {
+    ZG_REQUIRE(d.mixer >= ZG_LM_MIX_HGRN2 && d.mixer <= ZG_LM_MIX_WINDOW_LINEAR, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
     ZG_REQUIRE(d.heads >= 1 && d.dim >= 1 && d.vdim >= 1, ZG_ERR_ARG, "layer %zu: heads %d dim %d vdim %d", i, d.heads, d.dim, d.vdim);
-    if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_CHANNEL_DELTA)
+    if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_CHANNEL_DELTA || d.mixer == ZG_LM_MIX_WINDOW_LINEAR)
         ZG_REQUIRE(d.kv_heads >= 1 && d.heads % d.kv_heads == 0, ZG_ERR_ARG, "layer %zu: %d heads on %d key heads", i, d.heads, d.kv_heads);
     if (d.mixer == ZG_LM_MIX_PARALLEL) {
         ZG_REQUIRE(d.vdim % 2 == 0, ZG_ERR_ARG, "layer %zu: %d value channels per head cannot be rotated in pairs", i, d.vdim);
@@ -531,6 +624,13 @@ int check_layer(const zg_lm_layer& d, size_t i) {
                    ZG_ERR_ARG, "layer %zu: rotary scaling constants", i);
         ZG_REQUIRE(d.lru_width >= 1 && d.lru_blocks >= 1 && d.lru_width % d.lru_blocks == 0 && d.lru_conv >= 1 && d.lru_conv <= 16, ZG_ERR_ARG,
                    "layer %zu: recurrent unit of %d channels in %d blocks, %d taps", i, d.lru_width, d.lru_blocks, d.lru_conv);
+    } else if (d.mixer == ZG_LM_MIX_WINDOW_LINEAR) {
+        ZG_REQUIRE(flags & ZG_LM_SIDE_BY_SIDE, ZG_ERR_UNSUPPORTED, "layer %zu: the window + linear pair is built for side-by-side sublayers", i);
+        ZG_REQUIRE(d.window >= 0 && d.keep_first >= 0 && d.conv >= 0 && d.conv <= 16, ZG_ERR_ARG, "layer %zu: window %d, %d first tokens kept, %d taps", i,
+                   d.window, d.keep_first, d.conv);
+        ZG_REQUIRE(d.lin_heads >= 1 && d.lin_dim >= 1 && d.lin_vdim >= 1 && d.lin_dim <= 256, ZG_ERR_UNSUPPORTED,
+                   "layer %zu: linear attention of %d heads, %d key and %d value channels (at most 256 key channels)", i, d.lin_heads, d.lin_dim,
+                   d.lin_vdim);
     } else if (d.mixer == ZG_LM_MIX_CHANNEL_DELTA) {
         ZG_REQUIRE(d.conv >= 1 && d.conv <= 16 && d.decay_rank >= 1 && d.gate_rank >= 1, ZG_ERR_ARG, "layer %zu: %d taps, inner sizes %d and %d", i,
                    d.conv, d.decay_rank, d.gate_rank);
@@ -553,8 +653,17 @@ int check_layer(const zg_lm_layer& d, size_t i) {
     ZG_REQUIRE(d.ff == ZG_LM_FF_NONE || d.ff_width >= 1, ZG_ERR_ARG, "layer %zu: feed-forward width %d", i, d.ff_width);
     ZG_REQUIRE(d.ff != ZG_LM_FF_MOE || (d.experts >= 1 && d.experts <= 256 && d.top >= 1 && d.top <= d.experts), ZG_ERR_UNSUPPORTED,
                "layer %zu: %d experts, %d chosen (at most 256 experts)", i, d.experts, d.top);
-    ZG_REQUIRE((d.ff_act == ZG_LM_ACT_GLU_SILU || d.ff_act == ZG_LM_ACT_GELU) && (d.router == ZG_LM_ROUTE_SOFTMAX_ALL || d.router == ZG_LM_ROUTE_TOP_LOGITS),
+    ZG_REQUIRE(d.ff_act >= ZG_LM_ACT_GLU_SILU && d.ff_act <= ZG_LM_ACT_GLU_CLIPPED && d.router >= ZG_LM_ROUTE_SOFTMAX_ALL &&
+                   d.router <= ZG_LM_ROUTE_SIGMOID_INPUT,
                ZG_ERR_ARG, "layer %zu: expert activation %d, router rule %d", i, d.ff_act, d.router);
+    if (d.ff == ZG_LM_FF_MOE && !(flags & ZG_LM_SIDE_BY_SIDE))
+        ZG_REQUIRE(d.ff_act != ZG_LM_ACT_GLU_CLIPPED && d.router != ZG_LM_ROUTE_SIGMOID_INPUT && d.shared_width == 0, ZG_ERR_UNSUPPORTED,
+                   "layer %zu: the clipped activation, the input-weighted router and the shared expert are built for side-by-side sublayers", i);
+    if (d.ff == ZG_LM_FF_MOE && d.ff_act == ZG_LM_ACT_GLU_CLIPPED)
+        ZG_REQUIRE(d.ff_limit > 0.0f && (d.shared_width == 0 || d.shared_limit > 0.0f), ZG_ERR_ARG, "layer %zu: clip %g (shared expert: %g)", i, d.ff_limit,
+                   d.shared_limit);
+    ZG_REQUIRE(d.shared_width >= 0 && (d.shared_width == 0 || d.ff_act == ZG_LM_ACT_GLU_CLIPPED), ZG_ERR_UNSUPPORTED,
+               "layer %zu: a shared expert needs the clipped gated activation", i);
     return ZG_OK;
 }
 
@@ -572,7 +681,18 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
     const bool few = M <= kGemvMaxRows;
     const bool canon = g->canon >= 1;
     const bool readd = (g->cfg.flags & ZG_LM_LOOP_READD) && g->cfg.loop_times > 1;
-    ZG_TRY(launch_embed(g->embed, d_ids, g->x, readd ? g->x0 : nullptr, g->embed_scale, M, W, g->V, g->flag, s));
+    ZG_TRY(launch_embed(g->embed, d_ids, g->x, readd ? g->x0 : nullptr, g->embed_scale, M, W, g->V, g->flag, d_pos, g->pos_freq, s));
+    const bool side = g->side;
+    // side-by-side sublayers: the sums a layer leaves for the next layer's norm kernel to add (x += a + b + w * bias)
+    const float *pend_a = nullptr, *pend_b = nullptr, *pend_bias = nullptr;
+    float pend_w = 0.0f;
+    auto copy_trace = [&](int p) -> int {
+        if (g->trace && !capturing && (size_t)(p + 1) * M * W <= g->trace_floats) {
+            ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
+            ZG_HIP(hipStreamSynchronize(s));
+        }
+        return ZG_OK;
+    };
     // h + conv(h) of a sublayer's input, and the tail of the slots moved on
     auto input_conv = [&](const float* w, size_t off) -> int {
         ConvArgs c;
@@ -587,6 +707,11 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         const zg_lm_layer& d = L.d;
         const int H = d.heads, D = d.dim, Vd = d.vdim;
         bool hc_ready = false;  // one launch has done everything up to the mixer's input (decode steps)
+        if (side) {  // what the layer before left open, and both norms of this layer from one statistic
+            ZG_TRY(launch_norm_two(g->x, pend_a, pend_b, pend_bias, pend_w, L.norm1, d.ff != ZG_LM_FF_NONE ? L.norm2 : nullptr, eps, g->h, g->hc, M, W, s));
+            pend_a = pend_b = pend_bias = nullptr;
+            h_ready = true;
+        }
         if (canon && single && !h_ready)
             ZG_TRY(launch_norm_conv_single(g->x, ps.readd ? g->x0 : nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, L.norm1, eps, M, W, g->canon,
                                            L.canon1, g->seq_state + ps.canon1_off, g->seq_floats, d_slot, g->hc, s, &hc_ready));
@@ -609,7 +734,36 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         };
         Linear lin;
         bool mid_done = false;  // x, and the feed-forward's input in g->hc, are already there
-        if (d.mixer == ZG_LM_MIX_PARALLEL) {
+        if (d.mixer == ZG_LM_MIX_WINDOW_LINEAR) {
+            const int G = d.kv_heads, HD = H * D, GD = G * D, GV = G * Vd, CC = HD + GD + GV, HV = H * Vd;
+            const int HR = d.lin_heads, DR = d.lin_dim, VR = d.lin_vdim, HRD = HR * DR, HRV = HR * VR, NP = L.n_cat, OC = HV + HRV;
+            const int og = CC, orq = CC + HV, org = orq + 2 * HRD + HRV;  // columns of the left gate, the right q | k | v, the right gate
+            lin = Linear();
+            lin.A = hin; lin.lda = W; lin.B = L.wcat; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            // left: biases and convolutions of q | k | v at once, the whole-projection norms, keys and values into the cache
+            ConvArgs cv;
+            cv.in = g->proj; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = CC; cv.C = CC; cv.taps = std::max(1, d.conv); cv.w = L.convw;
+            cv.pre_bias = L.qkv_bias; cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
+            ZG_TRY(launch_causal_conv(cv, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+            ZG_TRY(launch_whole_norm_prep(g->ta, CC, M, HD, GD, GV, L.qnorm, L.knorm, eps, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
+            bool split = false;
+            ZG_TRY(launch_window_attention_split(g->ta, CC, g->o, OC, M, H, G, D, Vd, d.scale, d.window, d.keep_first, nullptr, nullptr, nullptr, d_pos,
+                                                 d_slot, g->page_table, g->max_pages, g->P, ps.cache,
+                                                 d.window > 0 ? d.window + d.keep_first : g->max_pages * g->P, g->win_ws, g->win_ws_floats, d_estart,
+                                                 d_elen, n_ent, s, &split));
+            if (!split)
+                ZG_TRY(launch_window_attention(g->ta, CC, g->o, OC, M, H, G, D, Vd, d.scale, d.window, d.keep_first, nullptr, nullptr, nullptr, d_pos,
+                                               d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
+            ZG_TRY(launch_norm_gate(g->o, OC, 1, HV, M, nullptr, eps, g->proj + og, NP, s, d.left_scale));
+            // right: the recurrence on silu(q | k | v), the heads normed together and gated
+            ZG_TRY(launch_hgrn2_scan(g->proj + orq, NP, g->o + HV, OC, g->seq_state + ps.rec_off, g->seq_floats, d_estart, d_elen, d_eslot, n_ent, M, HR,
+                                     DR, VR, nullptr, nullptr, g->scan_ws, g->scan_ws_floats, s, L.decay));
+            ZG_TRY(launch_norm_gate(g->o + HV, OC, 1, HRV, M, L.rnorm, eps, g->proj + org, NP, s, d.right_scale));
+            lin = Linear();  // both output projections at once: [c_l left | c_r right] against [left.o | right.o]
+            lin.A = g->o; lin.lda = OC; lin.B = L.ocat; lin.ldb = OC; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = OC;
+            ZG_TRY(launch_linear(lin, f32, s));
+        } else if (d.mixer == ZG_LM_MIX_PARALLEL) {
             const int G = d.kv_heads, C = d.lru_width, NB = d.lru_blocks, BS = C / NB, HV = H * Vd, NP = L.n_cat;
             const int oy = H * D + G * D + G * Vd, ox = oy + C;  // columns of the two branches of the recurrent unit
             const Rotary rot{L.rot_freq, d.rot_dims, 1.0f};
@@ -619,11 +773,11 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             // left: attention inside the window
             ZG_TRY(launch_window_prep(g->proj, NP, M, H, G, D, Vd, rot, L.vfreq, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
             bool split = false;
-            ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
+            ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, 0, L.sink, L.talk, L.vfreq, d_pos, d_slot,
                                                  g->page_table, g->max_pages, g->P, ps.cache, d.window > 0 ? d.window : g->max_pages * g->P, g->win_ws,
                                                  g->win_ws_floats, d_estart, d_elen, n_ent, s, &split));
             if (!split)
-                ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, L.sink, L.talk, L.vfreq, d_pos, d_slot,
+                ZG_TRY(launch_window_attention(g->proj, NP, g->o, HV, M, H, G, D, Vd, d.scale, d.window, 0, L.sink, L.talk, L.vfreq, d_pos, d_slot,
                                                g->page_table, g->max_pages, g->P, ps.cache, s));
             lin = Linear();
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
@@ -712,6 +866,72 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));
         }
+        if (side) {  // the feed-forward beside the mixer, on the second norm of the same x
+            const int F = d.ff_width;
+            const float* fin = g->hc;
+            if (d.ff == ZG_LM_FF_DENSE) {
+                lin = Linear();
+                lin.A = fin; lin.lda = W; lin.B = L.up; lin.ldb = W; lin.C = g->u; lin.ldc = F; lin.M = M; lin.N = F; lin.K = W; lin.act = ACT_RELU2;
+                ZG_TRY(launch_linear(lin, f32, s));
+                lin = Linear();
+                lin.A = g->u; lin.lda = F; lin.B = L.down; lin.ldb = F; lin.C = g->y2; lin.ldc = W; lin.M = M; lin.N = W; lin.K = F;
+                ZG_TRY(launch_linear(lin, f32, s));
+            } else if (d.ff == ZG_LM_FF_MOE) {
+                const int E = d.experts, top = d.top, NA = M * top;
+                const int UF = d.ff_act == ZG_LM_ACT_GELU ? F : 2 * F;
+                const bool on_input = d.router == ZG_LM_ROUTE_SIGMOID_INPUT;  // the router's score multiplies the expert's input
+                ZG_TRY(launch_route(fin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s));
+                Linear up, dn;
+                up.A = fin; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
+                up.N = UF; up.K = W;
+                if (d.ff_act == ZG_LM_ACT_GELU) up.act = ACT_GELU_ERF;
+                dn.A = g->hb; dn.lda = F; dn.B = L.edown; dn.ldb = F; dn.b_zoff = (long long)W * F; dn.C = g->ye; dn.ldc = W; dn.N = W; dn.K = F;
+                if (few) {  // one batch per assignment, its expert's matrices looked up on the device
+                    up.M = dn.M = 1; up.nz = dn.nz = NA; up.z_group = dn.z_group = g->pick;
+                    up.c_zoff = UF; dn.c_zoff = W;
+                } else {  // assignments sorted by expert, grouped products
+                    ZG_TRY(launch_group(g->pick, NA, E, g->grp_off, g->sorted, g->inv, s));
+                    up.M = dn.M = NA; up.a_rows = g->sorted; up.grp_off = dn.grp_off = g->grp_off; up.n_groups = dn.n_groups = E;
+                }
+                ZG_TRY(launch_linear(up, f32, s));
+                // (the product is linear: the score that multiplies an expert's input is applied to the product, in front of the clip)
+                if (d.ff_act == ZG_LM_ACT_GELU) {
+                    dn.A = g->gu_buf; dn.lda = F;
+                } else if (d.ff_act == ZG_LM_ACT_GLU_SILU) {
+                    ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
+                } else if (few) {  // the activation is applied where the second product reads its rows
+                    dn.A = g->gu_buf; dn.lda = 2 * F; dn.a_glu = F; dn.glu_kind = GLU_CLIPPED; dn.glu_limit = d.ff_limit;
+                    dn.glu_scale = on_input ? g->wt : nullptr;
+                } else {
+                    ZG_TRY(launch_glu_clipped(g->gu_buf, UF, g->hb, NA, F, d.ff_limit, on_input ? g->wt : nullptr, g->sorted, -1, s));
+                }
+                ZG_TRY(launch_linear(dn, f32, s));
+                const float* ys = nullptr;
+                if (d.shared_width > 0) {  // the shared expert; its gate logit is the last column of its first product
+                    const int S = d.shared_width;
+                    lin = Linear();
+                    lin.A = fin; lin.lda = W; lin.B = L.sgu; lin.ldb = W; lin.C = g->tb; lin.ldc = 2 * S + 1; lin.M = M; lin.N = 2 * S + 1; lin.K = W;
+                    ZG_TRY(launch_linear(lin, f32, s));
+                    ZG_TRY(launch_glu_clipped(g->tb, 2 * S + 1, g->tc, M, S, d.shared_limit, nullptr, nullptr, 2 * S, s));
+                    lin = Linear();
+                    lin.A = g->tc; lin.lda = S; lin.B = L.sdown; lin.ldb = S; lin.C = g->td; lin.ldc = W; lin.M = M; lin.N = W; lin.K = S;
+                    ZG_TRY(launch_linear(lin, f32, s));
+                    ys = g->td;
+                }
+                ZG_TRY(launch_expert_sum(g->y2, g->ye, few ? nullptr : g->inv, on_input ? nullptr : g->wt, top, ys, M, W, s));
+            }
+            pend_a = g->y;
+            pend_b = d.ff != ZG_LM_FF_NONE ? g->y2 : nullptr;
+            pend_bias = d.mixer == ZG_LM_MIX_WINDOW_LINEAR ? L.obias : nullptr;
+            pend_w = d.left_scale;
+            if (p + 1 == g->n_passes || (g->trace && !capturing)) {  // nobody behind to add them (or the stream is to be shown): add now
+                ZG_TRY(launch_add_two(g->x, pend_a, pend_b, pend_bias, pend_w, M, W, s));
+                pend_a = pend_b = pend_bias = nullptr;
+            }
+            ZG_TRY(copy_trace(p));
+            h_ready = false;
+            continue;
+        }
         if (canon && single && d.ff != ZG_LM_FF_NONE && !mid_done)
             ZG_TRY(launch_norm_conv_single(g->x, nullptr, g->y, nullptr, nullptr, nullptr, L.norm1b, L.norm2, eps, M, W, g->canon, L.canon2,
                                            g->seq_state + ps.canon2_off, g->seq_floats, d_slot, g->hc, s, &mid_done));
@@ -740,7 +960,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             const int E = d.experts, top = d.top, NA = M * top;
             const bool glu = d.ff_act == ZG_LM_ACT_GLU_SILU;
             const int UF = glu ? 2 * F : F;
-            ZG_TRY(launch_route(hin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router == ZG_LM_ROUTE_TOP_LOGITS, s));
+            ZG_TRY(launch_route(hin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s));
             Linear up, dn;
             up.A = hin; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
             up.N = UF; up.K = W;
@@ -765,13 +985,10 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             if (few) ZG_TRY(tail(nullptr, g->ye, g->wt, top, L.norm2b));
             if (!h_ready) ZG_TRY(launch_moe_combine(g->x, g->ye, few ? nullptr : g->inv, g->wt, top, L.norm2b, eps, M, W, s));
         }
-        if (g->trace && !capturing && (size_t)(p + 1) * M * W <= g->trace_floats) {
-            ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
-            ZG_HIP(hipStreamSynchronize(s));
-        }
+        ZG_TRY(copy_trace(p));
     }
     // the rows the last tokens of the entries left for the token shift of their successors
-    if (!canon) ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
+    if (!canon && !side) ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
 
     return ZG_OK;
 }
@@ -844,9 +1061,14 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             // so the twin is free again when the next batch fills it)
             for (int j = 0; j < nw; ++j) want_rows[j] = wants[w0 + j].first;
             ZG_HIP(hipMemcpyAsync(g->meta + 5 * (size_t)MS, want_rows, nw * sizeof(int), hipMemcpyHostToDevice, s));
-            ZG_TRY(launch_norm_gather(g->x, d_want, g->final_norm, eps, g->hn, nw, W, s));
+            ZG_TRY(launch_norm_gather(g->x, d_want, g->final_norm, eps, g->hn, nw, W, g->side, s));
             Linear lin;
             lin.A = g->hn; lin.lda = W; lin.B = g->head; lin.ldb = W; lin.C = g->logits; lin.ldc = g->V; lin.M = nw; lin.N = g->V; lin.K = W;
+            if ((g->cfg.logit_scale != 0.0f && g->cfg.logit_scale != 1.0f) || g->cfg.logit_softcap > 0.0f) {
+                lin.act = ACT_SCALE_SOFTCAP;
+                lin.act_a = g->cfg.logit_scale != 0.0f ? g->cfg.logit_scale : 1.0f;
+                lin.act_b = g->cfg.logit_softcap;
+            }
             ZG_TRY(launch_linear(lin, f32, s));
             if (sampler) {
                 ZG_TRY(launch_row_argmax(g->logits, nw, g->V, g->row_max, g->tok_out, g->amax_val, g->amax_idx, s));
@@ -955,12 +1177,12 @@ int step_impl(zg_lm* g, const zg_lm_entry* entries, size_t n_entries, float* log
             Slot& sl = g->slots[entries[i].seq];
             if (sl.len + 1 <= (size_t)g->keep_tokens) continue;
             const size_t dead = (sl.len + 1 - g->keep_tokens) / g->P;  // the next token sees positions >= len + 1 - keep
-            for (size_t pg = 0; pg < dead && pg < sl.pages.size(); ++pg)
+            for (size_t pg = g->keep_pages; pg < dead && pg < sl.pages.size(); ++pg)
                 if (sl.pages[pg] >= 0) {
                     g->free_pages.push_back(sl.pages[pg]);
                     sl.pages[pg] = -1;
                 }
-            sl.first_live = std::max(sl.first_live, std::min(dead, sl.pages.size()));
+            if (g->keep_pages == 0) sl.first_live = std::max(sl.first_live, std::min(dead, sl.pages.size()));
         }
     return ZG_OK;
 }
@@ -997,15 +1219,20 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     g->n_pages = g->max_pages + g->NS;  // every open sequence may leave one page partly used
     g->logit_rows = std::min(g->MS, 256);
     g->canon = config->canon_taps;
+    g->side = (config->flags & ZG_LM_SIDE_BY_SIDE) != 0;
     g->embed_scale = config->embed_scale != 0.0f ? config->embed_scale : 1.0f;
     int status = ZG_OK;
     for (size_t i = 0; i < config->n_layers && status == ZG_OK; ++i) {
-        status = check_layer(config->layers[i], i);
+        status = check_layer(config->layers[i], i, config->flags);
         LayerW L;
         L.d = config->layers[i];
         g->layers.push_back(L);
     }
     g->cfg.layers = nullptr;
+    if (status == ZG_OK && g->side && (g->canon != 0 || config->loop_times > 1)) {
+        set_error("lm_create: side-by-side sublayers have no input convolution and no looped span");
+        status = ZG_ERR_UNSUPPORTED;
+    }
     if (status == ZG_OK && (g->canon < 0 || g->canon > 16)) {
         set_error("lm_create: %d taps of the input convolution (0 to 16)", g->canon);
         status = ZG_ERR_ARG;
@@ -1045,8 +1272,20 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
             attends = true;
             g->keep_tokens = std::max(g->keep_tokens, d.window);
         }
+        if (d.mixer == ZG_LM_MIX_WINDOW_LINEAR) {
+            attends = true;
+            if (d.window > 0) {
+                g->keep_tokens = std::max(g->keep_tokens, d.window);
+                g->keep_first = std::max(g->keep_first, d.keep_first);
+            } else {
+                bounded = false;
+            }
+        }
     }
     if (!attends || !bounded) g->keep_tokens = 0;
+    // kept first tokens hold their pages for good: the pages between them and the window go back to the pool, but the page table
+    // cannot wrap round (a sequence is then bounded by the table: max_tokens)
+    g->keep_pages = g->keep_tokens > 0 ? (g->keep_first + g->P - 1) / g->P : 0;
     Bump measure{nullptr};
     layout(g, measure);
     g->arena_bytes = measure.off + 256;
@@ -1085,6 +1324,16 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
         const size_t nsq = (size_t)g->NS * g->seq_floats;
         zero_kernel<<<(unsigned)((nsq + 255) / 256), 256, 0, g->stream>>>(g->seq_state, nsq);
     }
+    if (g->pos_freq) {  // 10000^(-2i/W), rounded once
+        std::vector<float> pf((g->W + 1) / 2);
+        for (size_t i = 0; i < pf.size(); ++i) pf[i] = (float)pow(10000.0, -2.0 * (double)i / (double)g->W);
+        ZG_LM_TRY_HIP(hipMemcpy(g->pos_freq, pf.data(), pf.size() * sizeof(float), hipMemcpyHostToDevice));
+    }
+    for (LayerW& L : g->layers)
+        if (L.d.mixer == ZG_LM_MIX_WINDOW_LINEAR && L.d.conv == 0) {  // no convolution: one tap of weight one
+            const size_t n = (size_t)L.d.heads * L.d.dim + (size_t)L.d.kv_heads * (L.d.dim + L.d.vdim);
+            ones_kernel<<<(unsigned)((n + 255) / 256), 256, 0, g->stream>>>(L.convw, n);
+        }
     for (LayerW& L : g->layers)
         if (L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION || L.d.mixer == ZG_LM_MIX_PARALLEL) {
             std::vector<float> freq;
@@ -1151,7 +1400,9 @@ int zg_lm_load_tensor(zg_lm* g, const char* name, const float* data, size_t len)
         } else {
             for (size_t i = 0; i < len; ++i) tmp[i] = rne(data[i]);
         }
-        ZG_HIP(hipMemcpy(t.dev, tmp.data(), len * sizeof(bf16_t), hipMemcpyHostToDevice));
+        if (t.ld > 0 && t.ld != t.cols)
+            ZG_HIP(hipMemcpy2D(t.dev, t.ld * sizeof(bf16_t), tmp.data(), t.cols * sizeof(bf16_t), t.cols * sizeof(bf16_t), t.rows, hipMemcpyHostToDevice));
+        else ZG_HIP(hipMemcpy(t.dev, tmp.data(), len * sizeof(bf16_t), hipMemcpyHostToDevice));
     }
     t.loaded = true;
     return ZG_OK;
@@ -1180,7 +1431,7 @@ int zg_lm_init_random(zg_lm* g, uint64_t seed, float std_) {
         Tensor& t = kv.second;
         const size_t n = t.rows * t.cols;
         fill_kernel<<<(unsigned)((n + 255) / 256), 256, 0, g->stream>>>(t.dev, n, seed * 0x9E3779B97F4A7C15ULL + (++idx) * 0xD1B54A32D192ED03ULL, t.init,
-                                                                        std_);
+                                                                        std_, t.cols, t.ld > 0 ? t.ld : t.cols);
         ZG_HIP(hipGetLastError());
         t.loaded = true;
     }

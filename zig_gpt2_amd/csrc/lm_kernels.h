@@ -15,7 +15,9 @@ namespace zg {
 namespace lm {
 
 // ------------------------------------------------------------------------------------------------ linear maps
-enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_GELU_ERF = 2 };
+enum { ACT_NONE = 0, ACT_RELU2 = 1, ACT_GELU_ERF = 2, ACT_SCALE_SOFTCAP = 3 /* v <- v act_a, then act_b tanh(v / act_b) when act_b > 0 */ };
+// Gated activations of rows [gate (F) | up (F)] (GLU_CLIPPED: also a row factor and the clip `limit`)
+enum { GLU_SILU = 0 /* silu(gate) up */, GLU_CLIPPED = 1 /* g sigmoid(1.702 g) (u + 1), g = min(s gate, limit), u = clamp(s up, -limit, limit) */ };
 
 // C[m][n] = act( sum_k A[arow(m)][k] * B[n][k] )      for m < M, n < N
 //   arow(m) = a_rows ? a_rows[m] / a_div : m          (row gather: a token's row feeds each of its expert assignments)
@@ -34,7 +36,11 @@ struct Linear {
     int ldc = 0;
     int M = 0, N = 0, K = 0;
     int act = ACT_NONE;
-    int a_glu = 0;  // > 0 (row-vector kernel only): A rows are [gate (a_glu) | up (a_glu)] and enter as silu(gate) * up, K = a_glu
+    float act_a = 1.0f, act_b = 0.0f;  // constants of ACT_SCALE_SOFTCAP
+    int a_glu = 0;  // > 0 (row-vector kernel only): A rows are [gate (a_glu) | up (a_glu)] and enter through their gated activation, K = a_glu
+    int glu_kind = GLU_SILU;
+    float glu_limit = 0.0f;            // GLU_CLIPPED
+    const float* glu_scale = nullptr;  // GLU_CLIPPED, batched one-row form: factor of batch z's row (null: 1)
     int nz = 1;
     long long a_zoff = 0, b_zoff = 0, c_zoff = 0;
     const int* z_group = nullptr;
@@ -48,7 +54,10 @@ constexpr int kGemvMaxRows = 8;
 // ------------------------------------------------------------------------------------------------ norms, embedding, shift
 // x[m] = table[ids[m]] (bf16 -> fp32); an id outside [0, vocab) raises *flag (pinned or device int) and yields a zero row.
 // scale multiplies the row; x_copy (may be null) receives the same rows.
-int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, hipStream_t s);
+// pos_freq != null: the position's sinusoid vector is added: entry 2i = sin(row_pos[m] * pos_freq[i]), entry 2i + 1 = cos of that
+// angle (an fp32 product; pos_freq[i] = 10000^(-2i/W), rounded once on the host).
+int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, const int* row_pos,
+                 const float* pos_freq, hipStream_t s);
 // RMS norm with a weight stored as an offset from one, then the token shift:
 //   h[m] = x[m] / rms(x[m]) * (1 + w);   out[m] = h[m] + (h[prev(m)] - h[m]) * mu
 // prev(m) = row_prev[m] when >= 0, else the row kept for the slot: shift_state[row_slot[m]] (zeros for a new sequence).
@@ -70,8 +79,15 @@ int launch_norm_add_norm(float* x, const float* y, const float* wb, const float*
 int launch_sum_norm_shift(float* x, const float* y, const float* yexp, const float* weight, int top, const float* wb, const float* wn, const float* mu,
                           float eps, float* out, int M, int W, const int* row_slot, const float* shift_state, size_t slot_stride,
                           const int* row_entry_if_last, float* last_out, hipStream_t s, bool* taken);
-// out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for)
-int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s);
+// out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for; plain: * w)
+int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, bool plain, hipStream_t s);
+// Side-by-side sublayers: both read the same x through norms with plain weights, so one pass serves both:
+//   [x[m] += add_a[m] + add_b[m] + add_w * add_bias  (what the layer before left; any of them may be null)]
+//   ha[m] = x[m] / rms(x[m]) * wa;   hb[m] = x[m] / rms(x[m]) * wb   (hb / wb may be null)
+int launch_norm_two(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w, const float* wa, const float* wb, float eps,
+                    float* ha, float* hb, int M, int W, hipStream_t s);
+// x[m] += a[m] + b[m] + w * bias          (a, b, bias may be null)
+int launch_add_two(float* x, const float* a, const float* b, const float* bias, float w, int M, int W, hipStream_t s);
 // In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)
 int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s);
 
@@ -81,9 +97,11 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
 // Per entry e (rows ent_start[e] .. + ent_len[e]) and head: S <- diag(f_t) S + (1 - f_t) v_t^T, o_t = S^T q_t, token by token,
 // S = state[ent_slot[e]] ([H][D][V] fp32) read at the start and written back at the end.  out rows [H V], row stride ldo.
 // M: rows of the step.  ws (may be null): workspace for the chunk-parallel form of long steps, (M / 64 + n_entries) * (H D V + H D) floats.
+// decay != null: linear attention with one fixed decay per head on the same machinery — proj rows [q (H D) | k (H D) | v (H V)], all
+// three through silu on their way in:  S <- decay[h] S + k_t v_t^T, o_t = S^T q_t   (bias / low unused).
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
                       const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
-                      float* ws, size_t ws_floats, hipStream_t s);
+                      float* ws, size_t ws_floats, hipStream_t s, const float* decay = nullptr);
 
 // ------------------------------------------------------------------------------------------------ latent attention
 // Rotary table of one layer: freq[i] for the rot_dims / 2 pairs (YaRN blend applied on the host) and the amplitude factor.
@@ -151,9 +169,15 @@ int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, R
 // out[m][h] = turn_back_pos( sum_j w_h(j) value_(h / (H/G))(j) ),  w_h = sum_g talk[h][g] p_g,
 // p_g(j) = exp(s_g(j)) / (exp(sink_g) + sum_j' exp(s_g(j'))),  s_g(j) = scale q_g . k(j),  over the keys pos - window < j <= pos
 // (window 0: all j <= pos).  sink / talk may be null (no sink / no mix).
+// keep_first > 0: beyond the window the first keep_first positions of the sequence stay visible (a row's keys are then numbered
+// kept tokens first, then the window).  vfreq == null: values are cached unrotated and nothing is turned back.
 int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
-                            const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                            int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s);
+// The prep of attention without rotation whose q and k are normed over the whole projection: rows qkv [q (H D) | k (G D) | v (G V)];
+// q <- q / rms(q) * wq in place (rms over all H D entries), k / rms(k) * wk and v into the token's cache row [G D | G V].
+int launch_whole_norm_prep(float* qkv, int ld, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps, const int* row_pos,
+                           const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s);
 
 // The same with a row's keys split over up to kWinSplits workgroups and the scores kept in a workspace (three launches): what
 // steps of few rows need to fill the chip, and prompt portions to compute every score once.  key_capacity: the most keys a row
@@ -164,7 +188,7 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
 constexpr int kWinSplits = 64;
 size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_split_out);
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
-                                  const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                                  int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
                                   size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken);
 
@@ -187,18 +211,29 @@ int launch_delta_prep(float* qk, int ldqk, int G, int D, float* beta, int ldb, i
 int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const float* beta, int ldb, const float* dec, int ldd, float* out,
                       int ldo, int H, int G, int D, int V, float* state, size_t slot_stride, const int* ent_start, const int* ent_len,
                       const int* ent_slot, int n_entries, hipStream_t s);
-// In place over M * rows_per_m vectors of `width` floats: v / rms(v) * w * sigmoid(gate) (gate laid out like v, row stride ldg)
-int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s);
+// In place over M * rows_per_m vectors of `width` floats: v / rms(v) * w * sigmoid(gate) * factor (gate laid out like v, row stride
+// ldg).  w == null: no norm, the gate and the factor only.
+int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s,
+                     float factor = 1.0f);
 
 // ------------------------------------------------------------------------------------------------ mixture of experts
 // Per row: z = router . g (fp32), s = softmax(z), the `top` experts by s + correction (lowest index wins a tie), weights s.
 // top_logits: z += correction (a bias), the `top` largest z (lowest index wins a tie), weights = softmax over the chosen z.
+// rule ZG_LM_ROUTE_SIGMOID_INPUT: the `top` largest z (= the largest sigmoid scores; lowest index wins a tie), weights sigmoid(z).
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 bool top_logits, hipStream_t s);
+                 int rule, hipStream_t s);
 // Sort the M * top assignments by expert: grp_off[E + 1], sorted[p] = assignment at sorted position p, inv[a] = position of a.
 int launch_group(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv, hipStream_t s);
 // h[p][j] = silu(gu[p][j]) * gu[p][F + j]
 int launch_glu(const float* gu, float* h, int rows, int F, hipStream_t s);
+// h[p][j] = act(s gu[p][j], s gu[p][F + j]) * t,  act(g, u) = g' sigmoid(1.702 g') (u' + 1), g' = min(g, limit), u' = clamp(u, -limit, limit)
+//   s = row_scale ? row_scale[row_of ? row_of[p] : p] : 1   (the router's score of the assignment that sits at sorted place p)
+//   t = gate_col >= 0 ? sigmoid(gu[p][gate_col]) : 1        (a gate logit that the same product left in the row)
+// gu rows ld floats apart.
+int launch_glu_clipped(const float* gu, int ld, float* h, int rows, int F, float limit, const float* row_scale, const int* row_of, int gate_col,
+                       hipStream_t s);
+// y[m] = sum_k (weight ? weight[m top + k] : 1) * yexp[inv ? inv[m top + k] : m top + k] (+ ys[m]), in choice order
+int launch_expert_sum(float* y, const float* yexp, const int* inv, const float* weight, int top, const float* ys, int M, int W, hipStream_t s);
 // y = sum_k weight[m][k] * yexp[inv ? inv[m top + k] : m top + k];   x[m] += y / rms(y) * (1 + w)
 int launch_moe_combine(float* x, const float* yexp, const int* inv, const float* weight, int top, const float* w, float eps, int M, int W,
                        hipStream_t s);

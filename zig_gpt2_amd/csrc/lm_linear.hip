@@ -34,17 +34,35 @@ struct LinArgs {
     int lda, ldb, ldc;
     int M, N, K;
     int a_div, act, n_groups, a_glu;
+    float act_a, act_b;
+    int glu_kind;
+    float glu_limit;
+    const float* glu_scale;
     int a_vec, b_vec;  // 16-byte loads allowed (alignment of base, leading dimension and batch offsets)
 };
 
-__device__ __forceinline__ float apply_act(float v, int act) {
-    if (act == ACT_RELU2) {
+__device__ __forceinline__ float apply_act(float v, const LinArgs& p) {
+    const int act = p.act;
+    if (act == ACT_SCALE_SOFTCAP) {
+        v *= p.act_a;
+        if (p.act_b > 0.0f) v = p.act_b * tanhf(v / p.act_b);
+    } else if (act == ACT_RELU2) {
         v = fmaxf(v, 0.0f);
         v = v * v;
     } else if (act == ACT_GELU_ERF) {
         v = 0.5f * v * (1.0f + erff(v * 0.70710678118654752f));
     }
     return v;
+}
+
+// the gated activation of a [gate | up] row, applied where a product reads it (sc: the row's factor, clipped form only)
+__device__ __forceinline__ float glu_on_load(float g, float u, const LinArgs& p, float sc) {
+    if (p.glu_kind == GLU_CLIPPED) {
+        g = fminf(g * sc, p.glu_limit);
+        u = fminf(fmaxf(u * sc, -p.glu_limit), p.glu_limit);
+        return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + expf(-g)) * u;
 }
 
 // eight consecutive weights of row `w` from column k, zero beyond K
@@ -80,13 +98,16 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     const float* A = p.A + (long long)z * p.a_zoff;
     float* C = p.C + (long long)z * p.c_zoff;
     const float* arow[MR];
+    float asc[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         arow[m] = nullptr;
+        asc[m] = 1.0f;
         if (m < p.M) {
             const int rid = p.z_group ? z * p.M + m : m;
             const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
             arow[m] = A + (long long)src * p.lda;
+            if (p.a_glu > 0 && p.glu_scale) asc[m] = p.glu_scale[rid];
         }
     }
     const bool two = n0 + 1 < p.N;
@@ -115,10 +136,10 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
                 if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
                     const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, p.K, p.a_vec && p.a_glu % 4 == 0);
                     const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, p.K, p.a_vec && p.a_glu % 4 == 0);
-                    a0.x = a0.x / (1.0f + expf(-a0.x)) * u0.x; a0.y = a0.y / (1.0f + expf(-a0.y)) * u0.y;
-                    a0.z = a0.z / (1.0f + expf(-a0.z)) * u0.z; a0.w = a0.w / (1.0f + expf(-a0.w)) * u0.w;
-                    a1.x = a1.x / (1.0f + expf(-a1.x)) * u1.x; a1.y = a1.y / (1.0f + expf(-a1.y)) * u1.y;
-                    a1.z = a1.z / (1.0f + expf(-a1.z)) * u1.z; a1.w = a1.w / (1.0f + expf(-a1.w)) * u1.w;
+                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]); a0.y = glu_on_load(a0.y, u0.y, p, asc[m]);
+                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]); a0.w = glu_on_load(a0.w, u0.w, p, asc[m]);
+                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]); a1.y = glu_on_load(a1.y, u1.y, p, asc[m]);
+                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]); a1.w = glu_on_load(a1.w, u1.w, p, asc[m]);
                 }
                 av[u][0] = a0;
                 av[u][1] = a1;
@@ -144,8 +165,8 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     for (int m = 0; m < MR; ++m) {
         const float s0 = wave_allsum(acc0[m]), s1 = wave_allsum(acc1[m]);
         if (lane == 0 && m < p.M) {
-            C[(long long)m * p.ldc + n0] = apply_act(s0, p.act);
-            if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1, p.act);
+            C[(long long)m * p.ldc + n0] = apply_act(s0, p);
+            if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1, p);
         }
     }
 }
@@ -163,13 +184,16 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
     const float* A = p.A + (long long)z * p.a_zoff;
     float* C = p.C + (long long)z * p.c_zoff;
     const float* arow[MR];
+    float asc[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         arow[m] = nullptr;
+        asc[m] = 1.0f;
         if (m < p.M) {
             const int rid = p.z_group ? z * p.M + m : m;
             const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
             arow[m] = A + (long long)src * p.lda;
+            if (p.a_glu > 0 && p.glu_scale) asc[m] = p.glu_scale[rid];
         }
     }
     const bf16_t* w0 = B + (long long)n0 * p.ldb;
@@ -197,10 +221,10 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
                 if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
                     const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, k_hi, p.a_vec && p.a_glu % 4 == 0);
                     const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, k_hi, p.a_vec && p.a_glu % 4 == 0);
-                    a0.x = a0.x / (1.0f + expf(-a0.x)) * u0.x; a0.y = a0.y / (1.0f + expf(-a0.y)) * u0.y;
-                    a0.z = a0.z / (1.0f + expf(-a0.z)) * u0.z; a0.w = a0.w / (1.0f + expf(-a0.w)) * u0.w;
-                    a1.x = a1.x / (1.0f + expf(-a1.x)) * u1.x; a1.y = a1.y / (1.0f + expf(-a1.y)) * u1.y;
-                    a1.z = a1.z / (1.0f + expf(-a1.z)) * u1.z; a1.w = a1.w / (1.0f + expf(-a1.w)) * u1.w;
+                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]); a0.y = glu_on_load(a0.y, u0.y, p, asc[m]);
+                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]); a0.w = glu_on_load(a0.w, u0.w, p, asc[m]);
+                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]); a1.y = glu_on_load(a1.y, u1.y, p, asc[m]);
+                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]); a1.w = glu_on_load(a1.w, u1.w, p, asc[m]);
                 }
                 s0 = fmaf(a0.x, wa[u][0], s0); s1 = fmaf(a0.x, wb[u][0], s1);
                 s0 = fmaf(a0.y, wa[u][1], s0); s1 = fmaf(a0.y, wb[u][1], s1);
@@ -227,7 +251,7 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
     if (threadIdx.x < MR * 2) {
         const int m = threadIdx.x >> 1, c = threadIdx.x & 1;
         if (m < p.M && n0 + c < p.N)
-            C[(long long)m * p.ldc + n0 + c] = apply_act((s_part[0][m][c] + s_part[1][m][c]) + (s_part[2][m][c] + s_part[3][m][c]), p.act);
+            C[(long long)m * p.ldc + n0 + c] = apply_act((s_part[0][m][c] + s_part[1][m][c]) + (s_part[2][m][c] + s_part[3][m][c]), p);
     }
 }
 
@@ -407,7 +431,7 @@ __global__ __launch_bounds__(256) void lm_gemm_kernel(const LinArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int m = m0 + (wy * WT + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-                if (m < m_end) C[(long long)m * p.ldc + n] = apply_act(acc[i][j][e], p.act);
+                if (m < m_end) C[(long long)m * p.ldc + n] = apply_act(acc[i][j][e], p);
             }
         }
 }
@@ -423,6 +447,7 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
     p.lda = L.lda; p.ldb = L.ldb; p.ldc = L.ldc; p.M = L.M; p.N = L.N; p.K = L.K;
     p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0; p.a_glu = L.a_glu;
+    p.act_a = L.act_a; p.act_b = L.act_b; p.glu_kind = L.glu_kind; p.glu_limit = L.glu_limit; p.glu_scale = L.glu_scale;
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
     if (!L.grp_off && L.M <= kGemvMaxRows) {

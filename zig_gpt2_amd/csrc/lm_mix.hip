@@ -36,13 +36,18 @@ __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z));
 __device__ __forceinline__ float sigmoid_f(float z) { return 1.0f / (1.0f + expf(-z)); }
 
 __global__ __launch_bounds__(256) void embed_kernel(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int W, int vocab,
-                                                    int* flag) {
+                                                    int* flag, const int* row_pos, const float* pos_freq) {
     const int m = blockIdx.x, id = ids[m];
     const bool ok = id >= 0 && id < vocab;
     if (!ok && threadIdx.x == 0) *flag = 1;
     const bf16_t* row = table + (size_t)(ok ? id : 0) * W;
+    const float fpos = row_pos ? (float)row_pos[m] : 0.0f;
     for (int i = threadIdx.x; i < W; i += blockDim.x) {
-        const float v = ok ? __uint_as_float((uint32_t)row[i] << 16) * scale : 0.0f;
+        float v = ok ? __uint_as_float((uint32_t)row[i] << 16) * scale : 0.0f;
+        if (row_pos) {  // entries (2j, 2j + 1) = (sin, cos) of the fp32 product position x frequency j
+            const float a = fpos * pos_freq[i >> 1];
+            v += (i & 1) ? cosf(a) : sinf(a);
+        }
         x[(size_t)m * W + i] = v;
         if (x_copy) x_copy[(size_t)m * W + i] = v;
     }
@@ -244,12 +249,74 @@ __global__ __launch_bounds__(256) void sum_norm_shift_kernel(float* x, const flo
     }
 }
 
-__global__ __launch_bounds__(256) void norm_gather_kernel(const float* x, const int* rows, const float* w, float eps, float* out, int W) {
+__global__ __launch_bounds__(256) void norm_gather_kernel(const float* x, const int* rows, const float* w, float eps, float* out, int W, float one) {
     __shared__ float s_red[8];
     const int j = blockIdx.x;
     const float* xr = x + (size_t)rows[j] * W;
     const float r = row_inv_rms(xr, W, eps, s_red);
-    for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)j * W + i] = xr[i] * r * (1.0f + w[i]);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) out[(size_t)j * W + i] = xr[i] * r * (one + w[i]);
+}
+
+// Side-by-side sublayers: the residual sum the layer before left open, then the two norms of the same row from one statistic.
+// Rows of up to 256 * kRowRegs floats stay in registers between the statistic and the results.
+__global__ __launch_bounds__(256) void norm_two_kernel(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w,
+                                                       const float* wa, const float* wb, float eps, float* ha, float* hb, int W) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    float* xr = x + (size_t)m * W;
+    const bool adds = add_a || add_b || add_bias;
+    auto value = [&](int i) {
+        float v = xr[i];
+        if (add_a) v += add_a[(size_t)m * W + i];
+        if (add_b) v += add_b[(size_t)m * W + i];
+        if (add_bias) v = fmaf(add_w, add_bias[i], v);
+        return v;
+    };
+    if (W <= 256 * kRowRegs) {
+        float v[kRowRegs];
+        float ss = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            v[j] = i < W ? value(i) : 0.0f;
+            ss = fmaf(v[j], v[j], ss);
+        }
+        ss = block_allsum(ss, s_red);
+        const float r = 1.0f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+        for (int j = 0; j < kRowRegs; ++j) {
+            const int i = threadIdx.x + 256 * j;
+            if (i < W) {
+                if (adds) xr[i] = v[j];
+                ha[(size_t)m * W + i] = v[j] * r * wa[i];
+                if (hb) hb[(size_t)m * W + i] = v[j] * r * wb[i];
+            }
+        }
+        return;
+    }
+    float ss = 0.0f;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = value(i);
+        if (adds) xr[i] = v;  // (each thread reads back only what it wrote itself)
+        ss = fmaf(v, v, ss);
+    }
+    ss = block_allsum(ss, s_red);
+    const float r = 1.0f / sqrtf(ss / (float)W + eps);
+    for (int i = threadIdx.x; i < W; i += blockDim.x) {
+        const float v = xr[i];
+        ha[(size_t)m * W + i] = v * r * wa[i];
+        if (hb) hb[(size_t)m * W + i] = v * r * wb[i];
+    }
+}
+
+__global__ __launch_bounds__(256) void add_two_kernel(float* x, const float* a, const float* b, const float* bias, float w, size_t n, int W) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = x[i];
+    if (a) v += a[i];
+    if (b) v += b[i];
+    if (bias) v = fmaf(w, bias[i % W], v);
+    x[i] = v;
 }
 
 // one wave per (row, head) vector
@@ -290,10 +357,13 @@ __device__ __forceinline__ bool scan_find_chunk(int id, const int* ent_len, int 
     return false;
 }
 
-template <int G>
+// LIN: linear attention with a fixed decay per head on the same layout — the staged "gate" array holds silu(k), the weight of
+// the token's value in the state's row, and every row decays by decay[h]:  S <- decay S + k v^T  (q, k, v through silu).
+template <int G, bool LIN>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride,
                                                          const int* ent_start, const int* ent_len, const int* ent_slot, int n_entries, int H, int D,
-                                                         int V, int mode, int SB, float* wsB, float* wsA, const float* bias, const float* low) {
+                                                         int V, int mode, int SB, float* wsB, float* wsA, const float* bias, const float* low,
+                                                         const float* decay) {
     extern __shared__ __attribute__((aligned(16))) float s_scan[];
     constexpr int Dp = G * kScanRows;
     const int cols = blockDim.x / G;
@@ -316,6 +386,7 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
     }
     const int m0 = ent_start[e];
     const size_t head_floats = (size_t)D * V;
+    const float dec = LIN ? decay[h] : 0.0f;
     float* S_slot = state + (size_t)ent_slot[e] * slot_stride + (size_t)h * head_floats;
     float* S_ws = wsB ? wsB + ((size_t)blockIdx.x * H + h) * head_floats : nullptr;
     const float* S_in = mode == SCAN_DIRECT ? S_slot : mode == SCAN_C ? S_ws : nullptr;
@@ -333,18 +404,23 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
             const int tt = idx / Dp, i = idx % Dp;
             const float* row = proj + (size_t)(m0 + tb + tt) * ld;
             // the gates are activated on their way into the LDS: q = silu(.), f = low + (1 - low) sigmoid(. + bias)
-            float qv = 0.0f, fv = 1.0f;
+            float qv = 0.0f, fv = LIN ? 0.0f : 1.0f;
             if (i < D) {
-                const float l = low[h * D + i];
                 qv = silu_f(row[h * D + i]);
-                fv = l + (1.0f - l) * sigmoid_f(row[HD + h * D + i] + bias[h * D + i]);
+                if (LIN) {
+                    fv = silu_f(row[HD + h * D + i]);
+                } else {
+                    const float l = low[h * D + i];
+                    fv = l + (1.0f - l) * sigmoid_f(row[HD + h * D + i] + bias[h * D + i]);
+                }
             }
             sq[idx] = qv;
             sf[idx] = fv;
         }
         for (int idx = threadIdx.x; idx < nb * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = idx % cols;
-            sv[idx] = j0 + jj < V ? proj[(size_t)(m0 + tb + tt) * ld + 2 * HD + h * V + j0 + jj] : 0.0f;
+            const float vin = j0 + jj < V ? proj[(size_t)(m0 + tb + tt) * ld + 2 * HD + h * V + j0 + jj] : 0.0f;
+            sv[idx] = LIN ? silu_f(vin) : vin;
         }
         __syncthreads();
         for (int tt = 0; tt < nb; ++tt) {
@@ -359,9 +435,9 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int r = r4 * 4 + u;
-                    S[r] = fmaf(fv[u], S[r], (1.0f - fv[u]) * v);
+                    S[r] = LIN ? fmaf(dec, S[r], fv[u] * v) : fmaf(fv[u], S[r], (1.0f - fv[u]) * v);
                     o = fmaf(S[r], qv[u], o);
-                    if (mode == SCAN_A) A[r] *= fv[u];
+                    if (mode == SCAN_A) A[r] *= LIN ? dec : fv[u];
                 }
             }
             if (mode != SCAN_A) {
@@ -821,9 +897,10 @@ __global__ __launch_bounds__(256) void row_argmax_kernel(const float* logits, in
 
 }  // namespace
 
-int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, hipStream_t s) {
+int launch_embed(const bf16_t* table, const int* ids, float* x, float* x_copy, float scale, int M, int W, int vocab, int* flag, const int* row_pos,
+                 const float* pos_freq, hipStream_t s) {
     if (M <= 0) return ZG_OK;
-    embed_kernel<<<M, 256, 0, s>>>(table, ids, x, x_copy, scale, W, vocab, flag);
+    embed_kernel<<<M, 256, 0, s>>>(table, ids, x, x_copy, scale, W, vocab, flag, pos_freq ? row_pos : nullptr, pos_freq);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
@@ -871,9 +948,25 @@ int launch_sum_norm_shift(float* x, const float* y, const float* yexp, const flo
     return ZG_OK;
 }
 
-int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, hipStream_t s) {
+int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, bool plain, hipStream_t s) {
     if (n_rows <= 0) return ZG_OK;
-    norm_gather_kernel<<<n_rows, 256, 0, s>>>(x, rows, w, eps, out, W);
+    norm_gather_kernel<<<n_rows, 256, 0, s>>>(x, rows, w, eps, out, W, plain ? 0.0f : 1.0f);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_norm_two(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w, const float* wa, const float* wb, float eps,
+                    float* ha, float* hb, int M, int W, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    norm_two_kernel<<<M, 256, 0, s>>>(x, add_a, add_b, add_bias, add_w, wa, wb, eps, ha, wb ? hb : nullptr, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_add_two(float* x, const float* a, const float* b, const float* bias, float w, int M, int W, hipStream_t s) {
+    const size_t n = (size_t)M * W;
+    if (n == 0) return ZG_OK;
+    add_two_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, a, b, bias, w, n, W);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
@@ -888,7 +981,7 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
 
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
                       const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
-                      float* ws, size_t ws_floats, hipStream_t s) {
+                      float* ws, size_t ws_floats, hipStream_t s, const float* decay) {
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 16 * kScanRows, ZG_ERR_UNSUPPORTED, "hgrn2: %d key channels per head (at most %d)", D, 16 * kScanRows);
     int G = 1;
@@ -905,9 +998,15 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
     const bool chunked = M >= 4 * kScanChunk && ws && ws_floats >= need;
     float* wsB = chunked ? ws : nullptr;
     float* wsA = chunked ? ws + (size_t)max_chunks * head_floats : nullptr;
-#define ZG_SCAN(G_, grid_x, mode)                                                                                                                 \
-    hgrn2_scan_kernel<G_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start, ent_len, \
-                                                                                        ent_slot, n_entries, H, D, V, mode, SB, wsB, wsA, bias, low)
+#define ZG_SCAN_L(G_, LIN_, grid_x, mode)                                                                                                   \
+    hgrn2_scan_kernel<G_, LIN_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start,     \
+                                                                                              ent_len, ent_slot, n_entries, H, D, V, mode, SB, wsB, \
+                                                                                              wsA, bias, low, decay)
+#define ZG_SCAN(G_, grid_x, mode)                    \
+    do {                                             \
+        if (decay) ZG_SCAN_L(G_, true, grid_x, mode); \
+        else ZG_SCAN_L(G_, false, grid_x, mode);     \
+    } while (0)
 #define ZG_SCAN_G(grid_x, mode)                    \
     switch (G) {                                   \
         case 1: ZG_SCAN(1, grid_x, mode); break;   \
@@ -930,6 +1029,7 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
     ZG_HIP(hipGetLastError());
 #undef ZG_SCAN_G
 #undef ZG_SCAN
+#undef ZG_SCAN_L
     return ZG_OK;
 }
 

@@ -29,7 +29,9 @@ __device__ __forceinline__ float block_allsum(float v, float* s_red) {
 // top_logits: the correction is a bias of the logits, the largest logits are chosen and the weights are the softmax over the chosen
 // logits alone.
 __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
-                                                    int* pick, float* weight, int top_logits) {
+                                                    int* pick, float* weight, int rule) {
+    const bool top_logits = rule != 0;  // rules that choose by the logits themselves
+    const bool sigmoid_w = rule == 2;   // ... and weigh a chosen expert by sigmoid(z), nothing renormalised
     __shared__ float s_z[kMaxExperts];
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* row = g + (size_t)m * W;
@@ -74,7 +76,7 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
     for (int i = 0; i < 4; ++i) z[i] = lane + 64 * i < E ? s_z[lane + 64 * i] : -INFINITY;
     if (top_logits) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) ch[i] = lane + 64 * i < E ? z[i] + correction[lane + 64 * i] : -INFINITY;
+        for (int i = 0; i < 4; ++i) ch[i] = lane + 64 * i < E ? z[i] + (correction ? correction[lane + 64 * i] : 0.0f) : -INFINITY;
         float ek[4] = {0.0f, 0.0f, 0.0f, 0.0f};  // exp(z_k - z_0) of choice k on lane k % 64, slot k / 64
         float first = 0.0f;
         for (int k = 0; k < top; ++k) {
@@ -97,6 +99,7 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
                 for (int i = 0; i < 4; ++i)
                     if ((cand >> 6) == i) {
                         pick[(size_t)m * top + k] = cand;
+                        if (sigmoid_w) weight[(size_t)m * top + k] = 1.0f / (1.0f + expf(-ch[i]));
                         ch[i] = -INFINITY;
                     }
             }
@@ -106,6 +109,7 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
                     if ((k >> 6) == i) ek[i] = expf(wbest - first);
             }
         }
+        if (sigmoid_w) return;
         const float sum = wave_allsum((ek[0] + ek[1]) + (ek[2] + ek[3]));
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -187,6 +191,42 @@ __global__ __launch_bounds__(256) void glu_kernel(const float* gu, float* h, siz
     h[idx] = a / (1.0f + expf(-a)) * b;
 }
 
+// the clipped gated activation: the gate capped from above, the linear part clipped on both sides and lifted by one
+__device__ __forceinline__ float glu_clipped_f(float g, float u, float limit) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.0f + expf(-1.702f * g)) * (u + 1.0f);
+}
+
+__global__ __launch_bounds__(256) void glu_clipped_kernel(const float* gu, int ld, float* h, size_t n, int F, float limit, const float* row_scale,
+                                                          const int* row_of, int gate_col) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const size_t r = idx / F;
+    const int j = (int)(idx % F);
+    const float* row = gu + r * ld;
+    const float sc = row_scale ? row_scale[row_of ? row_of[r] : r] : 1.0f;
+    float v = glu_clipped_f(sc * row[j], sc * row[F + j], limit);
+    if (gate_col >= 0) v *= 1.0f / (1.0f + expf(-row[gate_col]));
+    h[idx] = v;
+}
+
+__global__ __launch_bounds__(256) void expert_sum_kernel(float* y, const float* yexp, const int* inv, const float* weight, int top, const float* ys,
+                                                         size_t n, int W) {
+    const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n) return;
+    const size_t m = idx / W;
+    const int i = (int)(idx % W);
+    float a = 0.0f;
+    for (int k = 0; k < top; ++k) {  // in choice order: the sum does not depend on the batch
+        const size_t as = m * top + k;
+        const float v = yexp[(size_t)(inv ? inv[as] : as) * W + i];
+        a = weight ? fmaf(weight[as], v, a) : a + v;
+    }
+    if (ys) a += ys[idx];
+    y[idx] = a;
+}
+
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* x, const float* yexp, const int* inv, const float* weight, int top, const float* w,
                                                           float eps, int W) {
     __shared__ float s_red[8];
@@ -212,11 +252,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* x, const float*
 }  // namespace
 
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 bool top_logits, hipStream_t s) {
+                 int rule, hipStream_t s) {
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(E >= 1 && E <= kMaxExperts && top >= 1 && top <= E, ZG_ERR_UNSUPPORTED, "router: %d experts, %d chosen (at most %d experts)", E, top,
                kMaxExperts);
-    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight, top_logits ? 1 : 0);
+    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight, rule);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
@@ -232,6 +272,23 @@ int launch_glu(const float* gu, float* h, int rows, int F, hipStream_t s) {
     const size_t n = (size_t)rows * F;
     if (n == 0) return ZG_OK;
     glu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gu, h, n, F);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_glu_clipped(const float* gu, int ld, float* h, int rows, int F, float limit, const float* row_scale, const int* row_of, int gate_col,
+                       hipStream_t s) {
+    const size_t n = (size_t)rows * F;
+    if (n == 0) return ZG_OK;
+    glu_clipped_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(gu, ld, h, n, F, limit, row_scale, row_of, gate_col);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_expert_sum(float* y, const float* yexp, const int* inv, const float* weight, int top, const float* ys, int M, int W, hipStream_t s) {
+    const size_t n = (size_t)M * W;
+    if (n == 0) return ZG_OK;
+    expert_sum_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(y, yexp, inv, weight, top, ys, n, W);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

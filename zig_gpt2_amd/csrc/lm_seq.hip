@@ -2,7 +2,8 @@
 //   * causal convolutions per channel whose last taps - 1 inputs live in a slot's state (the input convolution of a sublayer,
 //     the short convolutions in front of the recurrences),
 //   * softmax attention inside a sliding window over a paged cache of rotated keys and rotated VALUES, with a sink in the
-//     denominator and the heads' weights mixed by a matrix,
+//     denominator and the heads' weights mixed by a matrix; optionally the first tokens of a sequence stay visible behind the
+//     window, and values may be cached unrotated,
 //   * the real-gated linear recurrent unit (elementwise recurrence),
 //   * the gated delta rule with one decay per key channel (a matrix state per head).
 // Everything here is fp32 in both precision modes: positions, angles, scores, weights, gates, decays, recurrent states.
@@ -244,12 +245,27 @@ __global__ __launch_bounds__(256) void window_prep_kernel(float* proj, int ld, i
 // normalised weights, their mix over the heads, and the weighted sum of the values of the head's own key/value head.  The
 // result is turned back by the query's position and stored.  Tiles start at the first key of the window: the order of every
 // sum depends on the position alone.
+// The keys a row sees, numbered from 0: first the kept tokens that lie in front of its window (the first `keep` positions of the
+// sequence stay visible), then the window's keys up to the row's own position.  Every kernel below walks this numbering, so the
+// order of a row's sums depends on its position alone.
+struct KeySpan {
+    int j_lo, n_first, n_keys;
+};
+__device__ __forceinline__ KeySpan key_span(int pos, int window, int keep) {
+    KeySpan k;
+    k.j_lo = window > 0 ? max(0, pos - window + 1) : 0;
+    k.n_first = min(keep, k.j_lo);
+    k.n_keys = k.n_first + pos - k.j_lo + 1;
+    return k;
+}
+__device__ __forceinline__ int key_pos(const KeySpan& k, int n) { return n < k.n_first ? n : k.j_lo + (n - k.n_first); }
+
 constexpr int kWinTile = 64;
 constexpr int kWinMaxHeads = 64;
 constexpr int kWinAcc = 16;  // outputs per thread: H * V <= 256 * kWinAcc
 
 __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, int ldq, float* out, int ldo, int H, int G, int D, int V,
-                                                               float scale, int window, const float* sink, const float* talk,
+                                                               float scale, int window, int keep, const float* sink, const float* talk,
                                                                const float* vfreq, const int* row_pos, const int* row_slot,
                                                                const int* page_table, int max_pages, int page_tokens, const float* cache) {
     extern __shared__ __attribute__((aligned(16))) float s_win[];
@@ -263,8 +279,8 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
     const int m = blockIdx.x, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int pos = row_pos[m];
     const int* pages = page_table + (size_t)row_slot[m] * max_pages;
-    const int j_lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int n_keys = pos - j_lo + 1;
+    const KeySpan span = key_span(pos, window, keep);
+    const int n_keys = span.n_keys;
     const int rep = H / G;
     const size_t cstride = (size_t)G * (D + V);
     for (int i = tid; i < H * D; i += blockDim.x) s_q[i] = q[(size_t)m * ldq + i];
@@ -280,7 +296,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
     auto tile_scores = [&](int t0, int nt) {
         __syncthreads();
         if (tid < nt) {
-            const int j = j_lo + t0 + tid;
+            const int j = key_pos(span, t0 + tid);
             s_row[tid] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
         }
         __syncthreads();
@@ -349,6 +365,10 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
     const float fpos = (float)pos;
     for (int o = tid; o < H * V; o += blockDim.x) {  // turned back by the query's position
         const int i = o % V;
+        if (!vfreq) {
+            out[(size_t)m * ldo + o] = s_o[o];
+            continue;
+        }
         float sn, cs;
         sincosf(fpos * vfreq[i >> 1], &sn, &cs);
         const float own = s_o[o], other = s_o[o - i + (i ^ 1)];
@@ -366,11 +386,12 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
 // A share is ceil(keys of the row / splits) consecutive keys: the order of every sum depends on the position alone.
 constexpr int kMixTile = 32;
 
-__device__ __forceinline__ void window_range(int pos, int window, int n_split, int split, int& j_lo, int& k0, int& k1) {
-    j_lo = window > 0 ? max(0, pos - window + 1) : 0;
-    const int n_keys = pos - j_lo + 1, chunk = (n_keys + n_split - 1) / n_split;
-    k0 = min(n_keys, split * chunk);
-    k1 = min(n_keys, k0 + chunk);
+__device__ __forceinline__ KeySpan window_range(int pos, int window, int keep, int n_split, int split, int& k0, int& k1) {
+    const KeySpan span = key_span(pos, window, keep);
+    const int chunk = (span.n_keys + n_split - 1) / n_split;
+    k0 = min(span.n_keys, split * chunk);
+    k1 = min(span.n_keys, k0 + chunk);
+    return span;
 }
 
 constexpr int kScoreTile = 128;  // keys whose scores a workgroup holds in the LDS at a time
@@ -378,7 +399,7 @@ constexpr int kScoreKeys = 8;    // keys a wave has in flight
 
 template <int RPL>
 __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
-                                                            const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                            int keep, const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
                                                             int page_tokens, const float* cache, float* sc, int NK, float* st) {
     extern __shared__ __attribute__((aligned(16))) float s_sc[];
     float* s_q = s_sc;                     // [H][64 RPL] (zero beyond D)
@@ -388,8 +409,8 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int 
     __shared__ int s_row[kScoreTile];
     const int split = blockIdx.x, n_split = gridDim.x, m = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pos = row_pos[m];
-    int j_lo, k0, k1;
-    window_range(pos, window, n_split, split, j_lo, k0, k1);
+    int k0, k1;
+    const KeySpan span = window_range(pos, window, keep, n_split, split, k0, k1);
     const int* pages = page_table + (size_t)row_slot[m] * max_pages;
     const int rep = H / G;
     const size_t cstride = (size_t)G * (D + V);
@@ -406,7 +427,7 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int 
         const int nt = min(kScoreTile, k1 - t0);
         __syncthreads();  // the tile before has been consumed (and, the first time, q is staged)
         for (int i = threadIdx.x; i < nt; i += blockDim.x) {
-            const int j = j_lo + t0 + i;
+            const int j = key_pos(span, t0 + i);
             s_row[i] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
         }
         __syncthreads();
@@ -484,7 +505,7 @@ __device__ __forceinline__ bool rows_find_block(int id, const int* ent_len, int 
 
 template <int DH>
 __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
-                                                                 const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
+                                                                 int keep, const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
                                                                  const int* row_slot, const int* page_table, int max_pages, int page_tokens,
                                                                  const float* cache, float* sc, int NK) {
     int e, b;
@@ -492,15 +513,19 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, kh = lane >> 5;
     const int m0 = ent_start[e] + 32 * b, nrows = min(32, ent_len[e] - 32 * b);
     const int pos0 = row_pos[m0], pos_last = pos0 + nrows - 1;
-    const int ka = window > 0 ? max(0, pos0 - window + 1) : 0;
-    const int n_tiles = (pos_last - ka) / 32 + 1, units = n_tiles * G;
+    // the block's keys, numbered like a row's: the kept tokens in front of the FIRST row's window, then everything from there to
+    // the last row's position (a superset of every row's keys; each pair is masked by its own row's span below)
+    const KeySpan blk = key_span(pos0, window, keep);
+    const int n_blk = blk.n_first + pos_last - blk.j_lo + 1;
+    const int n_tiles = (n_blk - 1) / 32 + 1, units = n_tiles * G;
     const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
     const int rep = H / G, Dh = (D + 1) / 2;
     const size_t cstride = (size_t)G * (D + V);
     const bool vec = D % 8 == 0 && V % 4 == 0 && ldq % 4 == 0 && ((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(cache)) & 15) == 0;
     for (int u = blockIdx.y * 4 + wave; u < units; u += 4 * gridDim.y) {
         const int tile = u / G, g = u % G;
-        const int j = ka + 32 * tile + r;
+        const int nk = 32 * tile + r;                          // the key's number inside the block
+        const int j = nk < n_blk ? key_pos(blk, nk) : pos_last + 1;  // its position (beyond the block: none)
         float kreg[DH];
         {
             const int jc = min(j, pos_last);
@@ -540,8 +565,9 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
             for (int i = 0; i < 16; ++i) {
                 const int qi = 8 * (i >> 2) + 4 * kh + (i & 3);
                 const int pi = pos0 + qi;
-                const int jlo = window > 0 ? max(0, pi - window + 1) : 0;
-                if (qi < nrows && j <= pi && j >= jlo) sc[((size_t)(m0 + qi) * H + h) * NK + (j - jlo)] = acc[i] * scale;
+                const KeySpan sp = key_span(pi, window, keep);
+                if (qi < nrows && j <= pi && (j >= sp.j_lo || j < sp.n_first))
+                    sc[((size_t)(m0 + qi) * H + h) * NK + (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j)] = acc[i] * scale;
             }
         }
     }
@@ -549,10 +575,11 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
 
 // Per row and head the maximum and the sum of exp of the row's scores (a wave per head, its lanes over the keys), filed as the
 // statistics of share 0; the other shares are marked empty.
-__global__ __launch_bounds__(256) void window_stats_kernel(const float* sc, int NK, int H, int window, int n_split, const int* row_pos, float* st) {
+__global__ __launch_bounds__(256) void window_stats_kernel(const float* sc, int NK, int H, int window, int keep, int n_split, const int* row_pos,
+                                                           float* st) {
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int pos = row_pos[m];
-    const int n_keys = window > 0 ? min(pos + 1, window) : pos + 1;
+    const int n_keys = key_span(pos, window, keep).n_keys;
     for (int h = wave; h < H; h += 4) {
         const float* sr = sc + ((size_t)m * H + h) * NK;
         float mx = -INFINITY;
@@ -569,7 +596,7 @@ __global__ __launch_bounds__(256) void window_stats_kernel(const float* sc, int 
     }
 }
 
-__global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
+__global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, int V, int window, int keep, const float* sink, const float* talk,
                                                          const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
                                                          int page_tokens, const float* cache, const float* sc, int NK, const float* st,
                                                          float* po) {
@@ -582,8 +609,8 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
     __shared__ int s_row[kMixTile];
     const int split = blockIdx.x, n_split = gridDim.x, m = blockIdx.y, tid = threadIdx.x;
     const int pos = row_pos[m];
-    int j_lo, k0, k1;
-    window_range(pos, window, n_split, split, j_lo, k0, k1);
+    int k0, k1;
+    const KeySpan span = window_range(pos, window, keep, n_split, split, k0, k1);
     const int* pages = page_table + (size_t)row_slot[m] * max_pages;
     const int rep = H / G;
     const size_t cstride = (size_t)G * (D + V);
@@ -608,7 +635,7 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
         const int nt = min(kMixTile, k1 - t0);
         __syncthreads();
         if (tid < nt) {
-            const int j = j_lo + t0 + tid;
+            const int j = key_pos(span, t0 + tid);
             s_row[tid] = pages[(j / page_tokens) % max_pages] * page_tokens + j % page_tokens;
         }
         for (int idx = tid; idx < H * kMixTile; idx += blockDim.x) {
@@ -618,8 +645,11 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
         __syncthreads();
         for (int idx = tid; idx < H * kMixTile; idx += blockDim.x) {
             const int h = idx / kMixTile, jj = idx % kMixTile;
-            float wsum = 0.0f;
-            for (int g = 0; g < H; ++g) wsum = fmaf(s_talk[h * H + g], s_p[g * kMixTile + jj], wsum);
+            float wsum = s_p[idx];  // no mixing matrix: every head keeps its own weights
+            if (talk) {
+                wsum = 0.0f;
+                for (int g = 0; g < H; ++g) wsum = fmaf(s_talk[h * H + g], s_p[g * kMixTile + jj], wsum);
+            }
             s_w[idx] = wsum;
         }
         __syncthreads();
@@ -659,7 +689,7 @@ constexpr int kPvKeys = 16;
 constexpr int kPvUnits = 3;  // (head, channel tile) units a wave accumulates (few: two workgroups share a compute unit and hide each other's loads)
 constexpr int kPvHeads = 16; // most heads of this form (a pair's weights of all heads sit in registers)
 
-__global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int D, int V, int window, const float* sink, const float* talk,
+__global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int D, int V, int window, int keep, const float* sink, const float* talk,
                                                               const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
                                                               const int* row_slot, const int* page_table, int max_pages, int page_tokens,
                                                               const float* cache, const float* sc, int NK, const float* st, int n_split,
@@ -676,8 +706,9 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, kh = lane >> 5;
     const int m0 = ent_start[e] + 32 * b, nrows = min(32, ent_len[e] - 32 * b);
     const int pos0 = row_pos[m0], pos_last = pos0 + nrows - 1;
-    const int ka = window > 0 ? max(0, pos0 - window + 1) : 0;
-    const int n_tiles = (pos_last - ka) / kPvKeys + 1, per = (n_tiles + gridDim.y - 1) / gridDim.y;
+    const KeySpan blk = key_span(pos0, window, keep);  // the block's keys, numbered as in window_scores_mfma_kernel
+    const int n_blk = blk.n_first + pos_last - blk.j_lo + 1;
+    const int n_tiles = (n_blk - 1) / kPvKeys + 1, per = (n_tiles + gridDim.y - 1) / gridDim.y;
     const int t_lo = min(n_tiles, (int)blockIdx.y * per), t_hi = min(n_tiles, t_lo + per);
     const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
     const int rep = H / G, ctiles = (V + 31) / 32, units = H * ctiles;
@@ -702,20 +733,27 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
         for (int i = 0; i < 16; ++i) acc[u][i] = 0.0f;
     const int u0 = (blockIdx.z * 4 + wave) * kPvUnits;  // this wave's first unit
     for (int tile = t_lo; tile < t_hi; ++tile) {
-        const int j0 = ka + kPvKeys * tile;
+        const int n0 = kPvKeys * tile;
         __syncthreads();  // the tile before has been consumed (and, the first time, the statistics are staged)
         if (tid < kPvKeys) {
-            const int jc = min(j0 + tid, pos_last);
+            const int jc = n0 + tid < n_blk ? key_pos(blk, n0 + tid) : pos_last;
             s_row[tid] = pages[(jc / page_tokens) % max_pages] * page_tokens + jc % page_tokens;
         }
         for (int pr = tid; pr < 32 * kPvKeys; pr += blockDim.x) {
-            const int row = pr / kPvKeys, kk = pr % kPvKeys, j = j0 + kk, pi = pos0 + row;
-            const int jlo = window > 0 ? max(0, pi - window + 1) : 0;
-            const bool ok = row < nrows && j <= pi && j >= jlo;
+            const int row = pr / kPvKeys, kk = pr % kPvKeys, pi = pos0 + row;
+            const int j = n0 + kk < n_blk ? key_pos(blk, n0 + kk) : pos_last + 1;
+            const KeySpan sp = key_span(pi, window, keep);
+            const bool ok = row < nrows && j <= pi && (j >= sp.j_lo || j < sp.n_first);
             float p[kPvHeads];  // (registers: the loops over it are unrolled to the kernel's most heads)
-            const float* sr = sc + (size_t)(m0 + min(row, nrows - 1)) * H * NK + (ok ? j - jlo : 0);
+            const float* sr = sc + (size_t)(m0 + min(row, nrows - 1)) * H * NK + (ok ? (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j) : 0);
 #pragma unroll
             for (int g = 0; g < kPvHeads; ++g) p[g] = (ok && g < H) ? expf(sr[(size_t)g * NK] - s_M[row * H + g]) * s_iZ[row * H + g] : 0.0f;
+            if (!talk) {  // no mixing matrix: every head keeps its own weights
+#pragma unroll
+                for (int g = 0; g < kPvHeads; ++g)
+                    if (g < H) s_w[(g * 32 + row) * KP + kk] = p[g];
+                continue;
+            }
             for (int h = 0; h < H; ++h) {
                 float wsum = 0.0f;
 #pragma unroll
@@ -761,6 +799,15 @@ __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int 
     const int m = blockIdx.x;
     const float fpos = (float)row_pos[m];
     const float* base = po + (size_t)m * n_split * H * V;
+    if (!vfreq) {  // unrotated values: the shares added in order, nothing to turn back
+        for (int o = threadIdx.x; o < H * V; o += blockDim.x) {
+            float a = 0.0f;
+#pragma unroll 8
+            for (int s2 = 0; s2 < n_split; ++s2) a += base[(size_t)s2 * H * V + o];
+            out[(size_t)m * ldo + o] = a;
+        }
+        return;
+    }
     for (int p = threadIdx.x; p < H * V / 2; p += blockDim.x) {  // a pair of channels: (2i, 2i + 1) of a head
         float a = 0.0f, b = 0.0f;
 #pragma unroll 8
@@ -1001,17 +1048,43 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ld
 
 // one wave per (row, head) vector, in place: v / rms(v) * w * sigmoid(gate)
 __global__ __launch_bounds__(256) void norm_gate_kernel(float* v, int ld, int rows_per_m, int width, int n_vec, const float* w, float eps,
-                                                        const float* gate, int ldg) {
+                                                        const float* gate, int ldg, float factor) {
     const int vec = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (vec >= n_vec) return;
     const size_t m = vec / rows_per_m, hh = vec % rows_per_m;
     float* p = v + m * ld + hh * width;
     const float* gp = gate + m * ldg + hh * width;
+    if (!w) {  // the gate and the factor only
+        for (int i = lane; i < width; i += 64) p[i] = p[i] * sigmoid_f(gp[i]) * factor;
+        return;
+    }
     float ss = 0.0f;
     for (int i = lane; i < width; i += 64) ss = fmaf(p[i], p[i], ss);
     ss = wave_allsum(ss);
-    const float r = 1.0f / sqrtf(ss / (float)width + eps);
+    const float r = 1.0f / sqrtf(ss / (float)width + eps) * factor;
     for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i] * sigmoid_f(gp[i]);
+}
+
+// Attention without rotation whose q and k are normed over the WHOLE projection (all heads together): one workgroup per row.
+__global__ __launch_bounds__(256) void whole_norm_prep_kernel(float* qkv, int ld, int HD, int GD, int GV, const float* wq, const float* wk, float eps,
+                                                              const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                              int page_tokens, float* cache) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x;
+    const int pos = row_pos[m];
+    const int page = page_table[(size_t)row_slot[m] * max_pages + (pos / page_tokens) % max_pages];
+    float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)GD + GV);
+    float* q = qkv + (size_t)m * ld;
+    const float *k = q + HD, *v = k + GD;
+    float sq = 0.0f, sk = 0.0f;
+    for (int i = threadIdx.x; i < HD; i += blockDim.x) sq = fmaf(q[i], q[i], sq);
+    for (int i = threadIdx.x; i < GD; i += blockDim.x) sk = fmaf(k[i], k[i], sk);
+    sq = block_allsum(sq, s_red);
+    sk = block_allsum(sk, s_red);
+    const float rq = 1.0f / sqrtf(sq / (float)HD + eps), rk = 1.0f / sqrtf(sk / (float)GD + eps);
+    for (int i = threadIdx.x; i < HD; i += blockDim.x) q[i] = q[i] * rq * wq[i];
+    for (int i = threadIdx.x; i < GD; i += blockDim.x) crow[i] = k[i] * rk * wk[i];
+    for (int i = threadIdx.x; i < GV; i += blockDim.x) crow[GD + i] = v[i];
 }
 
 }  // namespace
@@ -1061,8 +1134,16 @@ int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, R
     return ZG_OK;
 }
 
+int launch_whole_norm_prep(float* qkv, int ld, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps, const int* row_pos,
+                           const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    whole_norm_prep_kernel<<<M, 256, 0, s>>>(qkv, ld, HD, GD, GV, wq, wk, eps, row_pos, row_slot, page_table, max_pages, page_tokens, cache);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
 int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
-                            const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                            int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s) {
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(H >= 1 && H <= kWinMaxHeads && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads on %d key heads (at most %d heads)",
@@ -1071,7 +1152,7 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
                256 * kWinAcc);
     const size_t lds = ((size_t)H * D + 2 * (size_t)H * kWinTile + (size_t)H * H + (size_t)H * V) * sizeof(float);
     ZG_REQUIRE(lds <= 60 * 1024, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads of %d + %d channels need %zu bytes of LDS", H, D, V, lds);
-    window_attention_kernel<<<M, 256, lds, s>>>(q, ldq, out, ldo, H, G, D, V, scale, window, sink, talk, vfreq, row_pos, row_slot, page_table,
+    window_attention_kernel<<<M, 256, lds, s>>>(q, ldq, out, ldo, H, G, D, V, scale, window, window > 0 ? keep_first : 0, sink, talk, vfreq, row_pos, row_slot, page_table,
                                                 max_pages, page_tokens, cache);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
@@ -1085,11 +1166,12 @@ size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_s
 }
 
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
-                                  const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
+                                  int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
                                   size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken) {
     *taken = false;
     if (M <= 0) return ZG_OK;
+    const int keep = window > 0 ? keep_first : 0;
     if (const char* e = getenv("ZGPT2_LM_WINDOW_GENERAL"))  // test hook: every step through the general kernel
         if (atoi(e) != 0) return ZG_OK;
     int n_split = 1;
@@ -1097,7 +1179,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     const int rpl = (D + 63) / 64;
     const size_t lds_a = ((size_t)H * 64 * rpl + (size_t)H * kScoreTile + 2 * (size_t)H) * sizeof(float);
     const size_t lds_b = (2 * (size_t)H * kMixTile + (size_t)H * H + 2 * (size_t)H) * sizeof(float);
-    if (!ws || need > ws_floats || H > kWinMaxHeads || H % G != 0 || H * V > 256 * kWinAcc || D > 256 || V % 2 != 0 || lds_a > 60 * 1024 ||
+    if (!ws || need > ws_floats || H > kWinMaxHeads || H % G != 0 || H * V > 256 * kWinAcc || D > 256 || (vfreq && V % 2 != 0) || lds_a > 60 * 1024 ||
         lds_b > 60 * 1024 || M > 65535)
         return ZG_OK;  // the general kernel takes it
     float* sc = ws;
@@ -1114,7 +1196,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
         const int ksplit = std::max(1, std::min(16, (max_tiles * G + 7) / 8));
         const dim3 tg((M + 31) / 32 + n_entries, ksplit);
 #define ZG_WT(R)                                                                                                                                   \
-    window_scores_mfma_kernel<R><<<tg, 256, 0, s>>>(q, ldq, H, G, D, V, scale, window, ent_start, ent_len, n_entries, row_pos, row_slot, page_table, \
+    window_scores_mfma_kernel<R><<<tg, 256, 0, s>>>(q, ldq, H, G, D, V, scale, window, keep, ent_start, ent_len, n_entries, row_pos, row_slot, page_table, \
                                                     max_pages, page_tokens, cache, sc, key_capacity)
         if (dh <= 8) ZG_WT(8);
         else if (dh <= 16) ZG_WT(16);
@@ -1122,11 +1204,11 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
         else ZG_WT(64);
 #undef ZG_WT
         ZG_HIP(hipGetLastError());
-        window_stats_kernel<<<M, 256, 0, s>>>(sc, key_capacity, H, window, n_split, row_pos, st);
+        window_stats_kernel<<<M, 256, 0, s>>>(sc, key_capacity, H, window, keep, n_split, row_pos, st);
         ZG_HIP(hipGetLastError());
     } else {
 #define ZG_WS(R)                                                                                                                              \
-    window_scores_kernel<R><<<grid, 256, lds_a, s>>>(q, ldq, H, G, D, V, scale, window, row_pos, row_slot, page_table, max_pages, page_tokens, cache, \
+    window_scores_kernel<R><<<grid, 256, lds_a, s>>>(q, ldq, H, G, D, V, scale, window, keep, row_pos, row_slot, page_table, max_pages, page_tokens, cache, \
                                                      sc, key_capacity, st)
     if (rpl <= 1) ZG_WS(1);
     else if (rpl <= 2) ZG_WS(2);
@@ -1138,10 +1220,10 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     if (tiled && H <= kPvHeads && lds_c <= 60 * 1024) {  // the value product of 32 rows at a time on the matrix cores
         const int units = H * ((V + 31) / 32);
         const dim3 pg((M + 31) / 32 + n_entries, n_split, (units + 4 * kPvUnits - 1) / (4 * kPvUnits));
-        window_mix_mfma_kernel<<<pg, 256, lds_c, s>>>(H, G, D, V, window, sink, talk, ent_start, ent_len, n_entries, row_pos, row_slot, page_table,
+        window_mix_mfma_kernel<<<pg, 256, lds_c, s>>>(H, G, D, V, window, keep, sink, talk, ent_start, ent_len, n_entries, row_pos, row_slot, page_table,
                                                       max_pages, page_tokens, cache, sc, key_capacity, st, n_split, po);
     } else {
-        window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
+        window_mix_kernel<<<grid, 256, lds_b, s>>>(H, G, D, V, window, keep, sink, talk, row_pos, row_slot, page_table, max_pages, page_tokens, cache, sc,
                                                    key_capacity, st, po);
     }
     ZG_HIP(hipGetLastError());
@@ -1199,10 +1281,11 @@ int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const 
     return ZG_OK;
 }
 
-int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s) {
+int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s,
+                     float factor) {
     const int n_vec = M * rows_per_m;
     if (n_vec <= 0) return ZG_OK;
-    norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg);
+    norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg, factor);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

@@ -15,6 +15,13 @@ config.json (zig_gpt2_amd/models.py maps architecture names to loaders; `DESIGNS
   head; the embedding output added again in front of every repetition of the loop but the first; plain gelu experts, the
   router's largest logits.  Sizes the configuration does not list (the inner sizes of two-step projections) come from the
   checkpoint's tensor shapes.
+  Sanazen: type "parallel" (mixer.left: grouped-query attention without rotation — q, k, v with biases through a short causal
+  convolution, q and k normed over the whole projection, a sliding window that keeps the first mask.keep_first tokens in sight,
+  heads gated by sigmoid(W_g h); mixer.right: linear attention with the fixed per-head `decay`; the branches summed with
+  left_scale / right_scale); a layer is x += mixer(norm1(x)) + mlp(norm2(x)) with plain norm weights; sinusoidal position
+  vectors added to the scaled embedding; experts with a clipped gated activation (`expert.limit`), chosen by their sigmoid
+  scores, the score multiplying the expert's input; mlp.shared: an expert every token uses, times sigmoid(shared.sg . h);
+  logit_scale, logit_softcap.
 """
 import ctypes as C
 import json
@@ -28,15 +35,20 @@ from . import _lib
 from ._lib import check_lm as check
 
 MIXERS = {"hgrn2": _lib.LM_MIX_HGRN2, "latent_attention": _lib.LM_MIX_LATENT_ATTENTION, "parallel": _lib.LM_MIX_PARALLEL,
-          "channel_delta": _lib.LM_MIX_CHANNEL_DELTA}
+          "channel_delta": _lib.LM_MIX_CHANNEL_DELTA, "window_linear": _lib.LM_MIX_WINDOW_LINEAR}
 ROT_STYLES = {"yarn": _lib.LM_ROT_YARN, "bands": _lib.LM_ROT_BANDS}
-EXPERT_ACTS = {"glu_silu": _lib.LM_ACT_GLU_SILU, "gelu": _lib.LM_ACT_GELU}
-ROUTERS = {"softmax_all": _lib.LM_ROUTE_SOFTMAX_ALL, "top_logits": _lib.LM_ROUTE_TOP_LOGITS}
+EXPERT_ACTS = {"glu_silu": _lib.LM_ACT_GLU_SILU, "gelu": _lib.LM_ACT_GELU, "glu_clipped": _lib.LM_ACT_GLU_CLIPPED}
+ROUTERS = {"softmax_all": _lib.LM_ROUTE_SOFTMAX_ALL, "top_logits": _lib.LM_ROUTE_TOP_LOGITS, "sigmoid_input": _lib.LM_ROUTE_SIGMOID_INPUT}
 
-# what an architecture name fixes beyond config.json
+# what an architecture name fixes beyond config.json.  mixers: layer type of config.json -> mixer of the library (two designs
+# call different pairs of branches "parallel")
 DESIGNS = {
-    "Tokosun": dict(mixers=("hgrn2", "latent_attention"), tied_head=False, loop_readd=False, expert_act="glu_silu", router="softmax_all"),
-    "Gupizen": dict(mixers=("parallel", "channel_delta"), tied_head=True, loop_readd=True, expert_act="gelu", router="top_logits"),
+    "Tokosun": dict(mixers={"hgrn2": "hgrn2", "latent_attention": "latent_attention"}, tied_head=False, loop_readd=False, expert_act="glu_silu",
+                    router="softmax_all"),
+    "Gupizen": dict(mixers={"parallel": "parallel", "channel_delta": "channel_delta"}, tied_head=True, loop_readd=True, expert_act="gelu",
+                    router="top_logits"),
+    "Sanazen": dict(mixers={"parallel": "window_linear"}, tied_head=False, loop_readd=False, expert_act="glu_clipped", router="sigmoid_input",
+                    side_by_side=True, sinusoid_positions=True),
 }
 
 
@@ -70,6 +82,16 @@ class LayerSpec:
     conv: int = 0
     decay_rank: int = 0
     gate_rank: int = 0
+    keep_first: int = 0
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    lin_heads: int = 0
+    lin_dim: int = 0
+    lin_vdim: int = 0
+    decay: Optional[list] = None  # one factor per head of the linear-attention branch
+    ff_limit: float = 0.0
+    shared_width: int = 0
+    shared_limit: float = 0.0
 
     @classmethod
     def from_json(cls, entry, design="Tokosun", shapes=None, prefix=""):
@@ -79,7 +101,20 @@ class LayerSpec:
         fixed = DESIGNS[design]
         if kind not in fixed["mixers"]:
             raise ValueError(f"unknown mixer type {kind!r} (known to {design}: {sorted(fixed['mixers'])})")
-        if kind == "parallel":
+        kind = fixed["mixers"][kind]
+        if kind == "window_linear":
+            l, r = m["left"], m["right"]
+            mask = l.get("mask") or {}
+            conv = l.get("conv")
+            if conv is None:  # the taps of the convolutions from the checkpoint; no such tensor: no convolution
+                conv = int(shapes[prefix + "mix.left.q.conv"][1]) if shapes and prefix + "mix.left.q.conv" in shapes else 0
+            kw = dict(mixer=kind, heads=int(l["heads"]), kv_heads=int(l.get("kv_heads", l["heads"])), dim=int(l["dim"]), vdim=int(l["vdim"]),
+                      scale=float(l["scale"]), window=int(mask.get("size", 0)), keep_first=int(mask.get("keep_first", 0)), conv=int(conv),
+                      left_scale=float(m.get("left_scale", 1.0)), right_scale=float(m.get("right_scale", 1.0)), lin_heads=int(r["heads"]),
+                      lin_dim=int(r["dim"]), lin_vdim=int(r["vdim"]), decay=[float(v) for v in r["decay"]])
+            if len(kw["decay"]) != kw["lin_heads"]:
+                raise ValueError(f"{prefix}mix.right: {len(kw['decay'])} decays for {kw['lin_heads']} heads")
+        elif kind == "parallel":
             l, r = m["left"], m["right"]
             rot = l.get("rot") or {}
             kw = dict(mixer=kind, heads=int(l["heads"]), kv_heads=int(l.get("kv_heads", l["heads"])), dim=int(l["dim"]), vdim=int(l["vdim"]),
@@ -110,6 +145,10 @@ class LayerSpec:
                 kw.update(ff="dense", ff_width=int(mlp["ff"]))
             elif mlp["kind"] == "moe":
                 kw.update(ff="moe", ff_width=int(mlp["expert"]["ff"]), experts=int(mlp["router"]["experts"]), top=int(mlp["router"]["top"]))
+                if fixed["expert_act"] == "glu_clipped":
+                    kw.update(ff_limit=float(mlp["expert"]["limit"]))
+                    if mlp.get("shared"):
+                        kw.update(shared_width=int(mlp["shared"]["ff"]), shared_limit=float(mlp["shared"]["limit"]))
             else:
                 raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
         return cls(**kw)
@@ -126,6 +165,12 @@ class LayerSpec:
             mixer = {"left": left, "right": {"width": self.lru_width, "blocks": self.lru_blocks, "conv": self.lru_conv}}
         elif self.mixer == "channel_delta":
             mixer.update(kv_heads=self.kv_heads, conv=self.conv, decay_rank=self.decay_rank, gate_rank=self.gate_rank)
+        elif self.mixer == "window_linear":
+            left = dict(mixer, kv_heads=self.kv_heads, scale=self.scale, conv=self.conv)
+            if self.window:
+                left["mask"] = {"size": self.window, "keep_first": self.keep_first}
+            mixer = {"left": left, "left_scale": self.left_scale, "right_scale": self.right_scale,
+                     "right": {"heads": self.lin_heads, "dim": self.lin_dim, "vdim": self.lin_vdim, "decay": list(self.decay)}}
         if self.mixer == "latent_attention":
             rot = {"base": self.rot_base, "dims": self.rot_dims}
             if self.rot_scaling:
@@ -136,7 +181,10 @@ class LayerSpec:
             mlp = {"kind": "dense", "ff": self.ff_width}
         elif self.ff == "moe":
             mlp = {"kind": "moe", "expert": {"ff": self.ff_width}, "router": {"experts": self.experts, "top": self.top}}
-        return {"type": self.mixer, "mixer": mixer, "mlp": mlp}
+            if self.expert_act == "glu_clipped":
+                mlp["expert"]["limit"] = self.ff_limit
+                mlp["shared"] = {"ff": self.shared_width, "limit": self.shared_limit} if self.shared_width else None
+        return {"type": "parallel" if self.mixer == "window_linear" else self.mixer, "mixer": mixer, "mlp": mlp}
 
     def to_c(self):
         sc = self.rot_scaling or {}
@@ -147,13 +195,16 @@ class LayerSpec:
                             float(sc.get("low" if bands else "slow", 1.0)),
                             {"none": _lib.LM_FF_NONE, "dense": _lib.LM_FF_DENSE, "moe": _lib.LM_FF_MOE}[self.ff], self.ff_width, self.experts,
                             self.top, self.kv_heads, self.window, self.lru_width, self.lru_blocks, self.lru_conv, self.conv, self.decay_rank,
-                            self.gate_rank, EXPERT_ACTS[self.expert_act], ROUTERS[self.router])
+                            self.gate_rank, EXPERT_ACTS[self.expert_act], ROUTERS[self.router], self.keep_first, self.left_scale, self.right_scale,
+                            self.lin_heads, self.lin_dim, self.lin_vdim, self.ff_limit, self.shared_width, self.shared_limit)
 
     def tensor_shapes(self, prefix, width, canon_taps=0):
         """{checkpoint tensor name: shape} of this layer."""
         H, D, V, W = self.heads, self.dim, self.vdim, width
         t = {prefix + "norm1": (W,), prefix + "norm1b": (W,)}
-        if canon_taps:
+        if self.mixer == "window_linear":  # plain norms in front of the sublayers only, nothing between norm and mixer
+            t = {prefix + "norm1": (W,)}
+        elif canon_taps:
             t[prefix + "canon1"] = (W, canon_taps)
             if self.ff != "none":
                 t[prefix + "canon2"] = (W, canon_taps)
@@ -167,6 +218,16 @@ class LayerSpec:
                       l + "out": (W,), r + "out": (W,), r + "y": (C, W), r + "y.b": (C,), r + "x": (C, W), r + "x.b": (C,),
                       r + "conv": (C, self.lru_conv), r + "conv.b": (C,), r + "ra": (NB, C // NB, C // NB), r + "ra.b": (NB, C // NB),
                       r + "ri": (NB, C // NB, C // NB), r + "ri.b": (NB, C // NB), r + "lam": (C,), r + "o": (W, C)})
+        elif self.mixer == "window_linear":
+            G, HR, DR, VR = self.kv_heads, self.lin_heads, self.lin_dim, self.lin_vdim
+            l, r = m + "left.", m + "right."
+            for u, n in (("q", H * D), ("k", G * D), ("v", G * V)):
+                t.update({l + u: (n, W), l + u + ".b": (n,)})
+                if self.conv:
+                    t[l + u + ".conv"] = (n, self.conv)
+            t.update({l + "q.norm": (H * D,), l + "k.norm": (G * D,), l + "g": (H * V, W), l + "o": (W, H * V), l + "o.b": (W,),
+                      r + "q": (HR * DR, W), r + "k": (HR * DR, W), r + "v": (HR * VR, W), r + "g": (HR * VR, W), r + "o": (W, HR * VR),
+                      r + "norm": (HR * VR,)})
         elif self.mixer == "channel_delta":
             G = self.kv_heads
             t.update({m + "q": (G * D, W), m + "q.conv": (G * D, self.conv), m + "k": (G * D, W), m + "k.conv": (G * D, self.conv),
@@ -183,15 +244,28 @@ class LayerSpec:
         f = prefix + "mlp."
         if self.ff != "none":
             t.update({prefix + "norm2": (W,), prefix + "norm2b": (W,)})
+            if self.mixer == "window_linear":
+                del t[prefix + "norm2b"]
         if self.ff == "dense":
             t.update({f + "up": (self.ff_width, W), f + "down": (W, self.ff_width)})
         elif self.ff == "moe":
             for e in range(self.experts):
                 t.update({f"{f}e{e}.up": (self.ff_width, W), f"{f}e{e}.down": (W, self.ff_width)})
-                if self.expert_act == "glu_silu":
+                if self.expert_act in ("glu_silu", "glu_clipped"):
                     t[f"{f}e{e}.gate"] = (self.ff_width, W)
-            t.update({f + "router": (self.experts, W), f + ("router.b" if self.router == "top_logits" else "correction"): (self.experts,)})
+            t[f + "router"] = (self.experts, W)
+            if self.router != "sigmoid_input":
+                t[f + ("router.b" if self.router == "top_logits" else "correction")] = (self.experts,)
+            if self.shared_width:
+                S = self.shared_width
+                t.update({f + "shared.gate": (S, W), f + "shared.up": (S, W), f + "shared.down": (W, S), f + "shared.sg": (1, W)})
         return t
+
+    def derived_tensors(self, prefix):
+        """{tensor name of the library: values} that the configuration holds instead of the checkpoint."""
+        if self.mixer == "window_linear":
+            return {prefix + "mix.right.decay": np.asarray(self.decay, np.float32)}
+        return {}
 
 
 @dataclass
@@ -204,6 +278,8 @@ class LMConfig:
     architecture: str = "Tokosun"
     embed_scale: float = 1.0
     canon_taps: int = 0  # > 0: both sublayers read h + conv(h) over this many tokens; 0: token shift in front of the mixer
+    logit_scale: float = 1.0
+    logit_softcap: float = 0.0  # > 0: logits <- cap tanh(logits / cap)
     extra: dict = field(default_factory=dict)
 
     @classmethod
@@ -215,7 +291,8 @@ class LMConfig:
         layers = [LayerSpec.from_json(e, arch, shapes, f"l{i}.") for i, e in enumerate(cfg["layers"])]
         return cls(vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers,
                    norm_eps=float(cfg["norm"]["eps"]), loop=dict(cfg["loop"]) if cfg.get("loop") else None, architecture=arch,
-                   embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), canon_taps=int((cfg.get("canon") or {}).get("taps", 0)))
+                   embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
+                   logit_scale=float(cfg.get("logit_scale") or 1.0), logit_softcap=float(cfg.get("logit_softcap") or 0.0))
 
     @classmethod
     def from_dir(cls, path):
@@ -234,6 +311,10 @@ class LMConfig:
             out["embedding"] = {"scale": self.embed_scale}
         if self.canon_taps:
             out["canon"] = {"taps": self.canon_taps}
+        if self.logit_scale != 1.0:
+            out["logit_scale"] = self.logit_scale
+        if self.logit_softcap:
+            out["logit_softcap"] = self.logit_softcap
         return out
 
     @property
@@ -242,7 +323,8 @@ class LMConfig:
 
     def flags(self):
         d = DESIGNS[self.architecture]
-        return (_lib.LM_TIED_HEAD if d["tied_head"] else 0) | (_lib.LM_LOOP_READD if d["loop_readd"] else 0)
+        return ((_lib.LM_TIED_HEAD if d["tied_head"] else 0) | (_lib.LM_LOOP_READD if d["loop_readd"] else 0) |
+                (_lib.LM_SIDE_BY_SIDE if d.get("side_by_side") else 0) | (_lib.LM_SINUSOID_POSITIONS if d.get("sinusoid_positions") else 0))
 
     def passes(self):
         """Layer index of every pass, in execution order."""
@@ -260,6 +342,13 @@ class LMConfig:
             t.update(l.tensor_shapes(f"l{i}.", self.width, self.canon_taps))
         return t
 
+    def derived_tensors(self):
+        """Tensors of the library that the configuration fills (constants listed per head), by name."""
+        t = {}
+        for i, l in enumerate(self.layers):
+            t.update(l.derived_tensors(f"l{i}."))
+        return t
+
 
 class LayeredLM:
     """A handle of the layered-model tier: weights, state slots, the step function and generation."""
@@ -275,10 +364,11 @@ class LayeredLM:
         cfg = _lib.LmConfig(config.vocab, config.width, len(config.layers), self._layers, int(loop["start"]), int(loop["stop"]), int(loop["times"]),
                             config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens,
                             (_lib.LM_F32 if dtype == "float32" else 0) | (0 if use_graph else _lib.LM_NO_GRAPH) | config.flags(),
-                            config.embed_scale, config.canon_taps)
+                            config.embed_scale, config.canon_taps, config.logit_scale, config.logit_softcap)
         h = C.c_void_p()
         check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
         self.h = h
+        self._load_derived()
         self.n_passes = len(config.passes())
         self.page_tokens = int(page_tokens) or 64  # (the library's default)
 
@@ -326,6 +416,11 @@ class LayeredLM:
             if missing:
                 raise KeyError(f"{len(missing)} tensors missing from the checkpoint: {' '.join(missing[:8])}")
 
+    def _load_derived(self):
+        for name, a in self.config.derived_tensors().items():
+            a = np.ascontiguousarray(a, dtype=np.float32)
+            check(self._L.zg_lm_load_tensor(self.h, name.encode(), a.ctypes.data, a.size))
+
     def missing_tensors(self):
         n, buf = C.c_size_t(), C.create_string_buffer(1 << 16)
         check(self._L.zg_lm_missing_tensors(self.h, C.byref(n), buf, len(buf)))
@@ -333,6 +428,7 @@ class LayeredLM:
 
     def init_random(self, seed=0, std=0.02):
         check(self._L.zg_lm_init_random(self.h, seed, std))
+        self._load_derived()
 
     # ------------------------------------------------------------------ sequences and steps
     def open(self):

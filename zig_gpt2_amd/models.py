@@ -35,6 +35,13 @@ def _load_gupizen(path, dtype="bfloat16", **kw):
     return lm.LayeredLM.from_dir(path, dtype=dtype, **kw)
 
 
+@register("Sanazen")
+def _load_sanazen(path, dtype="bfloat16", **kw):
+    from . import lm
+
+    return lm.LayeredLM.from_dir(path, dtype=dtype, **kw)
+
+
 @register("gpt2")
 def _load_gpt2(path, dtype="float32", config="124M", **kw):
     from . import gpt
