@@ -21,6 +21,7 @@ before left (None: the start of a sequence) and returns the new one.
 import numpy as np
 
 F = np.float64
+PROBE = None  # a list: every call of the left branch appends its softmax weights [heads, queries, keys] (for tests that build on them)
 
 
 def rms_unit(v, eps):
@@ -109,6 +110,8 @@ def gated_window_attention(h, w, p, m, eps, positions, state):
     k_pos = np.arange(keys.shape[0])
     ok = visible(positions, k_pos, int(mask.get("size", 0)), int(mask.get("keep_first", 0)))
     a = softmax_weights(q, keys, float(m["scale"]), ok, H, G)
+    if PROBE is not None:
+        PROBE.append(a)
     o = np.einsum("htn,nhv->thv", a, np.repeat(values, H // G, axis=1)).reshape(-1, H * V)
     o = o * sigmoid(h @ w[p + "g"].astype(F).T)
     return o @ w[p + "o"].astype(F).T + w[p + "o.b"].astype(F), st

@@ -155,12 +155,25 @@ inline Json safetensors_header(const std::string& path) {
 
 // config.json of a layered design -> layer descriptors (the keys zig_gpt2_amd/lm.py reads).  tensors: the checkpoint's
 // safetensors header, for the sizes that only a tensor's shape gives (may be null when the configuration lists them).
-inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm_layer>& layers, zg_lm_config& out) {
+// derived (may be null): tensors of the library that the configuration fills instead of the checkpoint (constants per head).
+typedef std::vector<std::pair<std::string, std::vector<float>>> DerivedTensors;
+inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm_layer>& layers, zg_lm_config& out, DerivedTensors* derived = nullptr) {
     const Json* arch = cfg.get("architecture");
     const std::string design = arch ? arch->str : std::string("?");
-    if (design != "Tokosun" && design != "Gupizen") throw std::runtime_error("config: architecture '" + design + "' is not served");
-    const bool gup = design == "Gupizen";
+    if (design != "Tokosun" && design != "Gupizen" && design != "Sanazen") throw std::runtime_error("config: architecture '" + design + "' is not served");
+    const bool gup = design == "Gupizen", san = design == "Sanazen";
     memset(&out, 0, sizeof(out));
+    if (san) {  // what the name fixes: side-by-side sublayers with plain norms, sinusoid positions
+        out.flags |= ZG_LM_SIDE_BY_SIDE | ZG_LM_SINUSOID_POSITIONS;
+        out.embed_scale = 1.0f;
+        if (const Json* e = cfg.get("embedding"))
+            if (e->truthy())
+                if (const Json* v = e->get("scale")) out.embed_scale = (float)v->num;
+        if (const Json* v = cfg.get("logit_scale"))
+            if (v->truthy()) out.logit_scale = (float)v->num;
+        if (const Json* v = cfg.get("logit_softcap"))
+            if (v->truthy()) out.logit_softcap = (float)v->num;
+    }
     if (gup) {  // what the name fixes: tied head, the embedding output added again per repetition of the loop
         out.flags |= ZG_LM_TIED_HEAD | ZG_LM_LOOP_READD;
         out.embed_scale = 1.0f;
@@ -188,7 +201,7 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
         const std::string& type = e.at("type").str;
         const Json& m = e.at("mixer");
         const std::string prefix = "l" + std::to_string(layer_index++) + ".";
-        const Json& sizes = (gup && type == "parallel") ? m.at("left") : m;
+        const Json& sizes = ((gup || san) && type == "parallel") ? m.at("left") : m;
         d.heads = (int)sizes.at("heads").num;
         d.dim = (int)sizes.at("dim").num;
         d.vdim = (int)sizes.at("vdim").num;
@@ -197,7 +210,35 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
             d.router = ZG_LM_ROUTE_TOP_LOGITS;
             d.kv_heads = sizes.get("kv_heads") ? (int)sizes.at("kv_heads").num : d.heads;
         }
-        if (gup && type == "parallel") {
+        if (san && type == "parallel") {
+            d.mixer = ZG_LM_MIX_WINDOW_LINEAR;
+            d.ff_act = ZG_LM_ACT_GLU_CLIPPED;
+            d.router = ZG_LM_ROUTE_SIGMOID_INPUT;
+            d.kv_heads = sizes.get("kv_heads") ? (int)sizes.at("kv_heads").num : d.heads;
+            d.scale = (float)sizes.at("scale").num;
+            if (const Json* mask = sizes.get("mask"))
+                if (mask->truthy()) {
+                    if (const Json* v = mask->get("size")) d.window = (int)v->num;
+                    if (const Json* v = mask->get("keep_first")) d.keep_first = (int)v->num;
+                }
+            if (const Json* v = sizes.get("conv")) {
+                d.conv = (int)v->num;
+            } else if (const Json* t = tensors ? tensors->get(prefix + "mix.left.q.conv") : nullptr) {  // the taps from the checkpoint
+                d.conv = (int)t->at("shape").arr.at(1).num;
+            }
+            d.left_scale = m.get("left_scale") ? (float)m.at("left_scale").num : 1.0f;
+            d.right_scale = m.get("right_scale") ? (float)m.at("right_scale").num : 1.0f;
+            const Json& r = m.at("right");
+            d.lin_heads = (int)r.at("heads").num;
+            d.lin_dim = (int)r.at("dim").num;
+            d.lin_vdim = (int)r.at("vdim").num;
+            std::vector<float> decay;
+            for (const Json& v : r.at("decay").arr) decay.push_back((float)v.num);
+            if ((int)decay.size() != d.lin_heads) throw std::runtime_error("config: " + prefix + "mix.right lists " + std::to_string(decay.size()) + " decays");
+            if (derived) derived->push_back({prefix + "mix.right.decay", decay});
+        } else if (san) {
+            throw std::runtime_error("config: unknown mixer type '" + type + "'");
+        } else if (gup && type == "parallel") {
             d.mixer = ZG_LM_MIX_PARALLEL;
             d.scale = (float)sizes.at("scale").num;
             if (const Json* mask = sizes.get("mask"))
@@ -271,6 +312,14 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
                 d.ff_width = (int)mlp->at("expert").at("ff").num;
                 d.experts = (int)mlp->at("router").at("experts").num;
                 d.top = (int)mlp->at("router").at("top").num;
+                if (san) {
+                    d.ff_limit = (float)mlp->at("expert").at("limit").num;
+                    const Json* sh = mlp->get("shared");
+                    if (sh && sh->truthy()) {
+                        d.shared_width = (int)sh->at("ff").num;
+                        d.shared_limit = (float)sh->at("limit").num;
+                    }
+                }
             } else {
                 throw std::runtime_error("config: unknown feed-forward kind '" + kind + "'");
             }
@@ -378,7 +427,8 @@ inline int lm_main(int argc, char** argv) {
         std::vector<zg_lm_layer> layers;
         zg_lm_config cfg;
         const Json tensors = safetensors_header(dir + "/model.safetensors");
-        build_config(JsonReader(slurp(dir + "/config.json")).parse(), &tensors, layers, cfg);
+        DerivedTensors derived;
+        build_config(JsonReader(slurp(dir + "/config.json")).parse(), &tensors, layers, cfg, &derived);
         size_t longest = 0, stride = 0;
         for (auto& pr : prompts) longest = std::max(longest, pr.size() + n_new), stride = std::max(stride, pr.size());
         cfg.max_seqs = prompts.size();
@@ -386,6 +436,9 @@ inline int lm_main(int argc, char** argv) {
         cfg.flags |= flags;
         zg_lm* g = nullptr;
         if (zg_lm_create(&g, &cfg, 0) != ZG_OK) throw std::runtime_error(std::string("create: ") + zg_last_error());
+        for (auto& kv : derived)
+            if (zg_lm_load_tensor(g, kv.first.c_str(), kv.second.data(), kv.second.size()) != ZG_OK)
+                throw std::runtime_error(std::string("load: ") + zg_last_error());
         load_safetensors(g, dir + "/model.safetensors");
         std::vector<int32_t> mat(prompts.size() * stride, 0), out(prompts.size() * n_new);
         std::vector<size_t> lens(prompts.size());
