@@ -48,9 +48,9 @@ def parse():
                    help="instead of the default workload: prompt and decode throughput of a layered model (Tokosun design, random weights) "
                         "at a size that resembles GPT-2 124M / medium / XL, beside the GPT-2 model of the same width and depth")
     p.add_argument("--lm-dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    p.add_argument("--lm-design", default="tokosun", choices=["tokosun", "gupizen"],
+    p.add_argument("--lm-design", default="tokosun", choices=["tokosun", "gupizen", "sanazen"],
                    help="with --lm: which design is measured.  gupizen: a Gupizen stack of the same width and depth, beside the Tokosun stack "
-                        "(the tier's closest model) instead of GPT-2")
+                        "(the tier's closest model) instead of GPT-2.  sanazen: a Sanazen stack beside the Gupizen stack of the same width and depth")
     p.add_argument("--dry-run", action="store_true",
                    help="CPU rehearsal of the launch path (gloo, no GPU, no kernels): rendezvous, prompt sharding, "
                         "weight-arena broadcast, barriers and the max-reduce; prints a line with dry_run=true")
@@ -463,6 +463,25 @@ def gupizen_bench_config(width, n_layers, vocab, window=512):
                        architecture="Gupizen", embed_scale=1.0, canon_taps=4)
 
 
+def sanazen_bench_config(width, n_layers, vocab, window=512):
+    """A Sanazen-design stack of `n_layers` window + linear-attention layers: attention heads of 64 channels on a quarter as many key
+    heads, a window of 512 tokens that keeps the first 4 in sight, convolutions of 4 taps; linear-attention heads of 128 x 128
+    (64 x 64 where the width does not divide) with decays from fast to slow; 8 clipped experts of width `width` of which 2 are
+    chosen, and a shared expert of the same width."""
+    from zig_gpt2_amd import lm
+
+    heads = width // 64
+    kv = heads // 4 if heads % 4 == 0 else heads // 5 if heads % 5 == 0 else heads
+    hd = 128 if width % 128 == 0 else 64
+    lh = width // hd
+    lay = dict(mixer="window_linear", heads=heads, kv_heads=kv, dim=64, vdim=64, scale=64 ** -0.5, window=window, keep_first=4, conv=4,
+               left_scale=1.0, right_scale=1.0, lin_heads=lh, lin_dim=hd, lin_vdim=hd, decay=[float(np.exp(-1.0 / (2.0 + 40.0 * i))) for i in range(lh)],
+               ff="moe", ff_width=width, experts=8, top=2, expert_act="glu_clipped", router="sigmoid_input", ff_limit=7.0, shared_width=width,
+               shared_limit=7.0)
+    return lm.LMConfig(vocab=vocab, width=width, layers=[lm.LayerSpec(**lay) for _ in range(n_layers)], norm_eps=1e-6, architecture="Sanazen",
+                       embed_scale=1.0, logit_scale=1.0, logit_softcap=30.0)
+
+
 def lm_weight_bytes(cfg):
     """(stored, read per decoded token) bytes of the bf16 matrices: every expert is stored, `top` of them are read."""
     stored = active = 0
@@ -488,6 +507,7 @@ def lm_bench(a):
     gcfg = synth.CONFIGS.get(gname) or synth.GPTConfig(50257, 1024, n_layers, width // 64, width)
     ctx = a.ctx or 1024
     gup = a.lm_design == "gupizen"
+    san = a.lm_design == "sanazen"
     cfg = lm_bench_config(width, n_layers, gcfg.vocab_size)
     out = {"metric": "lm_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.lm_dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, filled on the GPU)",
@@ -540,6 +560,15 @@ def lm_bench(a):
         m.close()
         return res
 
+    if san:  # beside the tier's closest model (attention in a window next to a recurrence, experts) at equal width and depth
+        s_res = measure(sanazen_bench_config(width, n_layers, gcfg.vocab_size))
+        g_res = measure(gupizen_bench_config(width, n_layers, gcfg.vocab_size))
+        d1 = s_res["decode"][0]
+        out["config"]["model"] = (f"Sanazen design, width {width}, {n_layers} layers (window 512 + 4 kept tokens beside linear attention; 8 experts, "
+                                  f"2 chosen, one shared), vocab {gcfg.vocab_size}")
+        out.update(value=d1["tokens_per_s"], ms_per_step=round(d1["wall_us_per_step"] / 1e3, 4), sanazen=s_res, gupizen_equal_size=g_res)
+        print(json.dumps(out))
+        return
     if gup:  # the new design beside the tier's closest model at equal width and depth
         g_res = measure(gupizen_bench_config(width, n_layers, gcfg.vocab_size))
         t_res = measure(lm_bench_config(width, n_layers, gcfg.vocab_size))
