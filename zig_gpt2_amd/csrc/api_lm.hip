@@ -683,9 +683,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
     const bool readd = (g->cfg.flags & ZG_LM_LOOP_READD) && g->cfg.loop_times > 1;
     ZG_TRY(launch_embed(g->embed, d_ids, g->x, readd ? g->x0 : nullptr, g->embed_scale, M, W, g->V, g->flag, d_pos, g->pos_freq, s));
     const bool side = g->side;
-    // side-by-side sublayers: the sums a layer leaves for the next layer's norm kernel to add (x += a + b + w * bias)
-    const float *pend_a = nullptr, *pend_b = nullptr, *pend_bias = nullptr;
-    float pend_w = 0.0f;
+    // side-by-side sublayers: the sums a layer leaves for the next layer's norm kernel to add
+    OpenSums pend;
     auto copy_trace = [&](int p) -> int {
         if (g->trace && !capturing && (size_t)(p + 1) * M * W <= g->trace_floats) {
             ZG_HIP(hipMemcpyAsync(g->trace + (size_t)p * M * W, g->x, (size_t)M * W * sizeof(float), hipMemcpyDeviceToHost, s));
@@ -708,8 +707,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         const int H = d.heads, D = d.dim, Vd = d.vdim;
         bool hc_ready = false;  // one launch has done everything up to the mixer's input (decode steps)
         if (side) {  // what the layer before left open, and both norms of this layer from one statistic
-            ZG_TRY(launch_norm_two(g->x, pend_a, pend_b, pend_bias, pend_w, L.norm1, d.ff != ZG_LM_FF_NONE ? L.norm2 : nullptr, eps, g->h, g->hc, M, W, s));
-            pend_a = pend_b = pend_bias = nullptr;
+            ZG_TRY(launch_norm_two(g->x, pend, L.norm1, d.ff != ZG_LM_FF_NONE ? L.norm2 : nullptr, eps, g->h, g->hc, M, W, s));
+            pend = OpenSums();
             h_ready = true;
         }
         if (canon && single && !h_ready)
@@ -745,17 +744,25 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             ConvArgs cv;
             cv.in = g->proj; cv.ld_in = NP; cv.out = g->ta; cv.ld_out = CC; cv.C = CC; cv.taps = std::max(1, d.conv); cv.w = L.convw;
             cv.pre_bias = L.qkv_bias; cv.tail = g->seq_state + ps.conv_off; cv.slot_stride = g->seq_floats;
-            ZG_TRY(launch_causal_conv(cv, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s));
-            ZG_TRY(launch_whole_norm_prep(g->ta, CC, M, HD, GD, GV, L.qnorm, L.knorm, eps, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
+            bool prepped = false;  // decode steps: convolution, norms and cache rows in one launch
+            if (single)
+                ZG_TRY(launch_conv_norm_prep_single(cv, g->ta, CC, M, HD, GD, GV, L.qnorm, L.knorm, eps, d_pos, d_slot, g->page_table, g->max_pages, g->P,
+                                                    ps.cache, s, &prepped));
+            if (!prepped) {
+                ZG_TRY(launch_causal_conv(cv, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s));
+                ZG_TRY(launch_whole_norm_prep(g->ta, CC, M, HD, GD, GV, L.qnorm, L.knorm, eps, d_pos, d_slot, g->page_table, g->max_pages, g->P, ps.cache,
+                                              s));
+            }
             bool split = false;
             ZG_TRY(launch_window_attention_split(g->ta, CC, g->o, OC, M, H, G, D, Vd, d.scale, d.window, d.keep_first, nullptr, nullptr, nullptr, d_pos,
                                                  d_slot, g->page_table, g->max_pages, g->P, ps.cache,
                                                  d.window > 0 ? d.window + d.keep_first : g->max_pages * g->P, g->win_ws, g->win_ws_floats, d_estart,
-                                                 d_elen, n_ent, s, &split));
-            if (!split)
+                                                 d_elen, n_ent, s, &split, g->proj + og, NP, d.left_scale));  // (the gate where the shares meet)
+            if (!split) {
                 ZG_TRY(launch_window_attention(g->ta, CC, g->o, OC, M, H, G, D, Vd, d.scale, d.window, d.keep_first, nullptr, nullptr, nullptr, d_pos,
                                                d_slot, g->page_table, g->max_pages, g->P, ps.cache, s));
-            ZG_TRY(launch_norm_gate(g->o, OC, 1, HV, M, nullptr, eps, g->proj + og, NP, s, d.left_scale));
+                ZG_TRY(launch_norm_gate(g->o, OC, 1, HV, M, nullptr, eps, g->proj + og, NP, s, d.left_scale));
+            }
             // right: the recurrence on silu(q | k | v), the heads normed together and gated
             ZG_TRY(launch_hgrn2_scan(g->proj + orq, NP, g->o + HV, OC, g->seq_state + ps.rec_off, g->seq_floats, d_estart, d_elen, d_eslot, n_ent, M, HR,
                                      DR, VR, nullptr, nullptr, g->scan_ws, g->scan_ws_floats, s, L.decay));
@@ -912,21 +919,34 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
                     lin = Linear();
                     lin.A = fin; lin.lda = W; lin.B = L.sgu; lin.ldb = W; lin.C = g->tb; lin.ldc = 2 * S + 1; lin.M = M; lin.N = 2 * S + 1; lin.K = W;
                     ZG_TRY(launch_linear(lin, f32, s));
-                    ZG_TRY(launch_glu_clipped(g->tb, 2 * S + 1, g->tc, M, S, d.shared_limit, nullptr, nullptr, 2 * S, s));
                     lin = Linear();
-                    lin.A = g->tc; lin.lda = S; lin.B = L.sdown; lin.ldb = S; lin.C = g->td; lin.ldc = W; lin.M = M; lin.N = W; lin.K = S;
+                    lin.B = L.sdown; lin.ldb = S; lin.C = g->td; lin.ldc = W; lin.M = M; lin.N = W; lin.K = S;
+                    if (few) {  // activation and gate where the second product reads its rows
+                        lin.A = g->tb; lin.lda = 2 * S + 1; lin.a_glu = S; lin.glu_kind = GLU_CLIPPED; lin.glu_limit = d.shared_limit; lin.glu_gate_col = 2 * S;
+                    } else {
+                        ZG_TRY(launch_glu_clipped(g->tb, 2 * S + 1, g->tc, M, S, d.shared_limit, nullptr, nullptr, 2 * S, s));
+                        lin.A = g->tc; lin.lda = S;
+                    }
                     ZG_TRY(launch_linear(lin, f32, s));
                     ys = g->td;
                 }
-                ZG_TRY(launch_expert_sum(g->y2, g->ye, few ? nullptr : g->inv, on_input ? nullptr : g->wt, top, ys, M, W, s));
+                if (few) {  // the experts' rows are added where the open sums are
+                    pend.exp = g->ye;
+                    pend.exp_w = on_input ? nullptr : g->wt;
+                    pend.top = top;
+                    pend.b = ys;
+                } else {
+                    ZG_TRY(launch_expert_sum(g->y2, g->ye, g->inv, on_input ? nullptr : g->wt, top, ys, M, W, s));
+                    pend.b = g->y2;
+                }
             }
-            pend_a = g->y;
-            pend_b = d.ff != ZG_LM_FF_NONE ? g->y2 : nullptr;
-            pend_bias = d.mixer == ZG_LM_MIX_WINDOW_LINEAR ? L.obias : nullptr;
-            pend_w = d.left_scale;
+            pend.a = g->y;
+            if (d.ff == ZG_LM_FF_DENSE) pend.b = g->y2;
+            pend.bias = d.mixer == ZG_LM_MIX_WINDOW_LINEAR ? L.obias : nullptr;
+            pend.w = d.left_scale;
             if (p + 1 == g->n_passes || (g->trace && !capturing)) {  // nobody behind to add them (or the stream is to be shown): add now
-                ZG_TRY(launch_add_two(g->x, pend_a, pend_b, pend_bias, pend_w, M, W, s));
-                pend_a = pend_b = pend_bias = nullptr;
+                ZG_TRY(launch_add_two(g->x, pend, M, W, s));
+                pend = OpenSums();
             }
             ZG_TRY(copy_trace(p));
             h_ready = false;

@@ -41,6 +41,7 @@ struct Linear {
     int glu_kind = GLU_SILU;
     float glu_limit = 0.0f;            // GLU_CLIPPED
     const float* glu_scale = nullptr;  // GLU_CLIPPED, batched one-row form: factor of batch z's row (null: 1)
+    int glu_gate_col = -1;             // >= 0: the activated row is multiplied by sigmoid(A row[glu_gate_col]) (a gate logit behind gate | up)
     int nz = 1;
     long long a_zoff = 0, b_zoff = 0, c_zoff = 0;
     const int* z_group = nullptr;
@@ -82,12 +83,19 @@ int launch_sum_norm_shift(float* x, const float* y, const float* yexp, const flo
 // out[j] = x[rows[j]] / rms * (1 + w)            (the model's last norm on the rows whose logits are asked for; plain: * w)
 int launch_norm_gather(const float* x, const int* rows, const float* w, float eps, float* out, int n_rows, int W, bool plain, hipStream_t s);
 // Side-by-side sublayers: both read the same x through norms with plain weights, so one pass serves both:
-//   [x[m] += add_a[m] + add_b[m] + add_w * add_bias  (what the layer before left; any of them may be null)]
+//   [x[m] += add.a[m] + add.b[m] + add.w * add.bias + sum_k (add.exp_w ? add.exp_w[m top + k] : 1) add.exp[m top + k]
+//    (what the layer before left open; any part may be null)]
 //   ha[m] = x[m] / rms(x[m]) * wa;   hb[m] = x[m] / rms(x[m]) * wb   (hb / wb may be null)
-int launch_norm_two(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w, const float* wa, const float* wb, float eps,
-                    float* ha, float* hb, int M, int W, hipStream_t s);
-// x[m] += a[m] + b[m] + w * bias          (a, b, bias may be null)
-int launch_add_two(float* x, const float* a, const float* b, const float* bias, float w, int M, int W, hipStream_t s);
+struct OpenSums {
+    const float *a = nullptr, *b = nullptr, *bias = nullptr;
+    float w = 0.0f;
+    const float *exp = nullptr, *exp_w = nullptr;  // rows of the chosen experts in assignment order, `top` per token
+    int top = 0;
+    __host__ __device__ bool any() const { return a || b || bias || exp; }
+};
+int launch_norm_two(float* x, const OpenSums& add, const float* wa, const float* wb, float eps, float* ha, float* hb, int M, int W, hipStream_t s);
+// x[m] += the same sums
+int launch_add_two(float* x, const OpenSums& add, int M, int W, hipStream_t s);
 // In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)
 int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s);
 
@@ -176,6 +184,11 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
                             const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s);
 // The prep of attention without rotation whose q and k are normed over the whole projection: rows qkv [q (H D) | k (G D) | v (G V)];
 // q <- q / rms(q) * wq in place (rms over all H D entries), k / rms(k) * wk and v into the token's cache row [G D | G V].
+// Steps of one row per entry: the convolution `a` over the channels q | k | v (its tails moved on) and the prep below in one launch,
+// q written normed to qout.  *taken = false (nothing launched) for rows beyond its registers.
+int launch_conv_norm_prep_single(const ConvArgs& a, float* qout, int ld_q, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps,
+                                 const int* row_pos, const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache,
+                                 hipStream_t s, bool* taken);
 int launch_whole_norm_prep(float* qkv, int ld, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps, const int* row_pos,
                            const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s);
 
@@ -190,7 +203,9 @@ size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_s
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                                   int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
-                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken);
+                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken,
+                                  const float* out_gate = nullptr, int ld_gate = 0, float out_factor = 1.0f);
+// (out_gate != null: a taken step multiplies the result by sigmoid(out_gate[m][.]) * out_factor where the shares are added)
 
 // ------------------------------------------------------------------------------------------------ real-gated linear recurrent unit
 // Per entry and channel c: r = sigmoid(gr + br), i = sigmoid(gi + bi), a = exp(-8 r softplus(lam)), S = a S + sqrt(1 - a^2) i u,

@@ -38,6 +38,7 @@ struct LinArgs {
     int glu_kind;
     float glu_limit;
     const float* glu_scale;
+    int glu_gate_col;
     int a_vec, b_vec;  // 16-byte loads allowed (alignment of base, leading dimension and batch offsets)
 };
 
@@ -98,16 +99,17 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
     const float* A = p.A + (long long)z * p.a_zoff;
     float* C = p.C + (long long)z * p.c_zoff;
     const float* arow[MR];
-    float asc[MR];
+    float asc[MR], agate[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         arow[m] = nullptr;
-        asc[m] = 1.0f;
+        asc[m] = agate[m] = 1.0f;
         if (m < p.M) {
             const int rid = p.z_group ? z * p.M + m : m;
             const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
             arow[m] = A + (long long)src * p.lda;
             if (p.a_glu > 0 && p.glu_scale) asc[m] = p.glu_scale[rid];
+            if (p.a_glu > 0 && p.glu_gate_col >= 0) agate[m] = 1.0f / (1.0f + expf(-arow[m][p.glu_gate_col]));
         }
     }
     const bool two = n0 + 1 < p.N;
@@ -136,10 +138,10 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
                 if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
                     const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, p.K, p.a_vec && p.a_glu % 4 == 0);
                     const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, p.K, p.a_vec && p.a_glu % 4 == 0);
-                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]); a0.y = glu_on_load(a0.y, u0.y, p, asc[m]);
-                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]); a0.w = glu_on_load(a0.w, u0.w, p, asc[m]);
-                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]); a1.y = glu_on_load(a1.y, u1.y, p, asc[m]);
-                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]); a1.w = glu_on_load(a1.w, u1.w, p, asc[m]);
+                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]) * agate[m]; a0.y = glu_on_load(a0.y, u0.y, p, asc[m]) * agate[m];
+                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]) * agate[m]; a0.w = glu_on_load(a0.w, u0.w, p, asc[m]) * agate[m];
+                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]) * agate[m]; a1.y = glu_on_load(a1.y, u1.y, p, asc[m]) * agate[m];
+                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]) * agate[m]; a1.w = glu_on_load(a1.w, u1.w, p, asc[m]) * agate[m];
                 }
                 av[u][0] = a0;
                 av[u][1] = a1;
@@ -184,16 +186,17 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
     const float* A = p.A + (long long)z * p.a_zoff;
     float* C = p.C + (long long)z * p.c_zoff;
     const float* arow[MR];
-    float asc[MR];
+    float asc[MR], agate[MR];
 #pragma unroll
     for (int m = 0; m < MR; ++m) {
         arow[m] = nullptr;
-        asc[m] = 1.0f;
+        asc[m] = agate[m] = 1.0f;
         if (m < p.M) {
             const int rid = p.z_group ? z * p.M + m : m;
             const int src = (p.a_rows ? p.a_rows[rid] : rid) / p.a_div;
             arow[m] = A + (long long)src * p.lda;
             if (p.a_glu > 0 && p.glu_scale) asc[m] = p.glu_scale[rid];
+            if (p.a_glu > 0 && p.glu_gate_col >= 0) agate[m] = 1.0f / (1.0f + expf(-arow[m][p.glu_gate_col]));
         }
     }
     const bf16_t* w0 = B + (long long)n0 * p.ldb;
@@ -221,10 +224,10 @@ __global__ __launch_bounds__(256) void lm_gemv_ks_kernel(const LinArgs p) {
                 if (p.a_glu > 0 && arow[m]) {  // rows [gate | up]: silu(gate) * up
                     const f32x4 u0 = load_a4(arow[m] + p.a_glu, kk, k_hi, p.a_vec && p.a_glu % 4 == 0);
                     const f32x4 u1 = load_a4(arow[m] + p.a_glu, kk + 4, k_hi, p.a_vec && p.a_glu % 4 == 0);
-                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]); a0.y = glu_on_load(a0.y, u0.y, p, asc[m]);
-                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]); a0.w = glu_on_load(a0.w, u0.w, p, asc[m]);
-                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]); a1.y = glu_on_load(a1.y, u1.y, p, asc[m]);
-                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]); a1.w = glu_on_load(a1.w, u1.w, p, asc[m]);
+                    a0.x = glu_on_load(a0.x, u0.x, p, asc[m]) * agate[m]; a0.y = glu_on_load(a0.y, u0.y, p, asc[m]) * agate[m];
+                    a0.z = glu_on_load(a0.z, u0.z, p, asc[m]) * agate[m]; a0.w = glu_on_load(a0.w, u0.w, p, asc[m]) * agate[m];
+                    a1.x = glu_on_load(a1.x, u1.x, p, asc[m]) * agate[m]; a1.y = glu_on_load(a1.y, u1.y, p, asc[m]) * agate[m];
+                    a1.z = glu_on_load(a1.z, u1.z, p, asc[m]) * agate[m]; a1.w = glu_on_load(a1.w, u1.w, p, asc[m]) * agate[m];
                 }
                 s0 = fmaf(a0.x, wa[u][0], s0); s1 = fmaf(a0.x, wb[u][0], s1);
                 s0 = fmaf(a0.y, wa[u][1], s0); s1 = fmaf(a0.y, wb[u][1], s1);
@@ -448,6 +451,7 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.lda = L.lda; p.ldb = L.ldb; p.ldc = L.ldc; p.M = L.M; p.N = L.N; p.K = L.K;
     p.a_div = L.a_div; p.act = L.act; p.n_groups = L.grp_off ? L.n_groups : 0; p.a_glu = L.a_glu;
     p.act_a = L.act_a; p.act_b = L.act_b; p.glu_kind = L.glu_kind; p.glu_limit = L.glu_limit; p.glu_scale = L.glu_scale;
+    p.glu_gate_col = L.glu_gate_col;
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
     if (!L.grp_off && L.M <= kGemvMaxRows) {

@@ -259,19 +259,29 @@ __global__ __launch_bounds__(256) void norm_gather_kernel(const float* x, const 
 
 // Side-by-side sublayers: the residual sum the layer before left open, then the two norms of the same row from one statistic.
 // Rows of up to 256 * kRowRegs floats stay in registers between the statistic and the results.
-__global__ __launch_bounds__(256) void norm_two_kernel(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w,
-                                                       const float* wa, const float* wb, float eps, float* ha, float* hb, int W) {
+__device__ __forceinline__ float open_sums_at(const OpenSums& add, size_t m, int i, int W, float v) {
+    if (add.a) v += add.a[m * W + i];
+    if (add.exp) {  // in choice order: the sum does not depend on the batch
+        float e = 0.0f;
+        for (int k = 0; k < add.top; ++k) {
+            const float y = add.exp[(m * add.top + k) * W + i];
+            e = add.exp_w ? fmaf(add.exp_w[m * add.top + k], y, e) : e + y;
+        }
+        v += add.b ? e + add.b[m * W + i] : e;
+    } else if (add.b) {
+        v += add.b[m * W + i];
+    }
+    if (add.bias) v = fmaf(add.w, add.bias[i], v);
+    return v;
+}
+
+__global__ __launch_bounds__(256) void norm_two_kernel(float* x, const OpenSums add, const float* wa, const float* wb, float eps, float* ha, float* hb,
+                                                       int W) {
     __shared__ float s_red[8];
     const int m = blockIdx.x;
     float* xr = x + (size_t)m * W;
-    const bool adds = add_a || add_b || add_bias;
-    auto value = [&](int i) {
-        float v = xr[i];
-        if (add_a) v += add_a[(size_t)m * W + i];
-        if (add_b) v += add_b[(size_t)m * W + i];
-        if (add_bias) v = fmaf(add_w, add_bias[i], v);
-        return v;
-    };
+    const bool adds = add.any();
+    auto value = [&](int i) { return adds ? open_sums_at(add, (size_t)m, i, W, xr[i]) : xr[i]; };
     if (W <= 256 * kRowRegs) {
         float v[kRowRegs];
         float ss = 0.0f;
@@ -309,14 +319,10 @@ __global__ __launch_bounds__(256) void norm_two_kernel(float* x, const float* ad
     }
 }
 
-__global__ __launch_bounds__(256) void add_two_kernel(float* x, const float* a, const float* b, const float* bias, float w, size_t n, int W) {
+__global__ __launch_bounds__(256) void add_two_kernel(float* x, const OpenSums add, size_t n, int W) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
-    float v = x[i];
-    if (a) v += a[i];
-    if (b) v += b[i];
-    if (bias) v = fmaf(w, bias[i % W], v);
-    x[i] = v;
+    x[i] = open_sums_at(add, i / W, (int)(i % W), W, x[i]);
 }
 
 // one wave per (row, head) vector
@@ -955,18 +961,17 @@ int launch_norm_gather(const float* x, const int* rows, const float* w, float ep
     return ZG_OK;
 }
 
-int launch_norm_two(float* x, const float* add_a, const float* add_b, const float* add_bias, float add_w, const float* wa, const float* wb, float eps,
-                    float* ha, float* hb, int M, int W, hipStream_t s) {
+int launch_norm_two(float* x, const OpenSums& add, const float* wa, const float* wb, float eps, float* ha, float* hb, int M, int W, hipStream_t s) {
     if (M <= 0) return ZG_OK;
-    norm_two_kernel<<<M, 256, 0, s>>>(x, add_a, add_b, add_bias, add_w, wa, wb, eps, ha, wb ? hb : nullptr, W);
+    norm_two_kernel<<<M, 256, 0, s>>>(x, add, wa, wb, eps, ha, wb ? hb : nullptr, W);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
 
-int launch_add_two(float* x, const float* a, const float* b, const float* bias, float w, int M, int W, hipStream_t s) {
+int launch_add_two(float* x, const OpenSums& add, int M, int W, hipStream_t s) {
     const size_t n = (size_t)M * W;
-    if (n == 0) return ZG_OK;
-    add_two_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, a, b, bias, w, n, W);
+    if (n == 0 || !add.any()) return ZG_OK;
+    add_two_kernel<<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, add, n, W);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

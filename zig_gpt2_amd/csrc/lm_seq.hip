@@ -794,8 +794,9 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
     }
 }
 
+// gate != null: the heads' outputs are multiplied by sigmoid(gate[m][.]) * factor on their way out (a gated attention's last step)
 __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int n_split, float* out, int ldo, int H, int V, const float* vfreq,
-                                                           const int* row_pos) {
+                                                           const int* row_pos, const float* gate, int ldg, float factor) {
     const int m = blockIdx.x;
     const float fpos = (float)row_pos[m];
     const float* base = po + (size_t)m * n_split * H * V;
@@ -804,6 +805,7 @@ __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int 
             float a = 0.0f;
 #pragma unroll 8
             for (int s2 = 0; s2 < n_split; ++s2) a += base[(size_t)s2 * H * V + o];
+            if (gate) a *= sigmoid_f(gate[(size_t)m * ldg + o]) * factor;
             out[(size_t)m * ldo + o] = a;
         }
         return;
@@ -817,8 +819,13 @@ __global__ __launch_bounds__(256) void window_merge_kernel(const float* po, int 
         }
         float sn, cs;
         sincosf(fpos * vfreq[p % (V / 2)], &sn, &cs);
-        out[(size_t)m * ldo + 2 * p] = a * cs + b * sn;
-        out[(size_t)m * ldo + 2 * p + 1] = b * cs - a * sn;
+        float oa = a * cs + b * sn, ob = b * cs - a * sn;
+        if (gate) {
+            oa *= sigmoid_f(gate[(size_t)m * ldg + 2 * p]) * factor;
+            ob *= sigmoid_f(gate[(size_t)m * ldg + 2 * p + 1]) * factor;
+        }
+        out[(size_t)m * ldo + 2 * p] = oa;
+        out[(size_t)m * ldo + 2 * p + 1] = ob;
     }
 }
 
@@ -1065,6 +1072,73 @@ __global__ __launch_bounds__(256) void norm_gate_kernel(float* v, int ld, int ro
     for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i] * sigmoid_f(gp[i]);
 }
 
+// the same for wide vectors: a workgroup per vector
+__global__ __launch_bounds__(256) void norm_gate_wide_kernel(float* v, int ld, int rows_per_m, int width, const float* w, float eps, const float* gate,
+                                                             int ldg, float factor) {
+    __shared__ float s_red[8];
+    const size_t m = blockIdx.x / rows_per_m, hh = blockIdx.x % rows_per_m;
+    float* p = v + m * ld + hh * width;
+    const float* gp = gate + m * ldg + hh * width;
+    float r = factor;
+    if (w) {
+        float ss = 0.0f;
+        for (int i = threadIdx.x; i < width; i += blockDim.x) ss = fmaf(p[i], p[i], ss);
+        ss = block_allsum(ss, s_red);
+        r = 1.0f / sqrtf(ss / (float)width + eps) * factor;
+    }
+    for (int i = threadIdx.x; i < width; i += blockDim.x) p[i] = p[i] * r * (w ? w[i] : 1.0f) * sigmoid_f(gp[i]);
+}
+
+// Decode steps (one row per entry) of the attention below: biases, the short convolutions of q | k | v with their tails moved
+// on, both whole-projection norms, q written normed, keys and values into the cache — one launch; a row's channels (up to
+// 256 * kPrepRegs) stay in registers between the convolution and the norms.
+constexpr int kPrepRegs = 16;
+__global__ __launch_bounds__(256) void conv_norm_prep_single_kernel(const float* in, int ld_in, float* qout, int ld_q, int HD, int GD, int GV, int taps,
+                                                                    const float* cw, const float* pre_bias, float* tail, size_t slot_stride,
+                                                                    const float* wq, const float* wk, float eps, const int* row_pos,
+                                                                    const int* row_slot, const int* page_table, int max_pages, int page_tokens,
+                                                                    float* cache) {
+    __shared__ float s_red[8];
+    const int m = blockIdx.x, CC = HD + GD + GV, K = taps - 1;
+    const int pos = row_pos[m], slot = row_slot[m];
+    const int page = page_table[(size_t)slot * max_pages + (pos / page_tokens) % max_pages];
+    float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)GD + GV);
+    float* tl = tail + (size_t)slot * slot_stride;
+    float val[kPrepRegs];
+    float sq = 0.0f, sk = 0.0f;
+#pragma unroll
+    for (int r = 0; r < kPrepRegs; ++r) {
+        const int c = threadIdx.x + 256 * r;
+        val[r] = 0.0f;
+        if (c < CC) {
+            const float cur = in[(size_t)m * ld_in + c] + (pre_bias ? pre_bias[c] : 0.0f);
+            float tv[kMaxTaps];
+#pragma unroll
+            for (int j = 0; j < kMaxTaps; ++j) tv[j] = j < K ? tl[(size_t)j * CC + c] : 0.0f;
+            float acc = cw[(size_t)c * taps + K] * cur;
+#pragma unroll
+            for (int j = 0; j < kMaxTaps; ++j)
+                if (j < K) acc = fmaf(cw[(size_t)c * taps + j], tv[j], acc);
+#pragma unroll
+            for (int j = 0; j < kMaxTaps; ++j)
+                if (j < K) tl[(size_t)j * CC + c] = j + 1 < K ? tv[min(j + 1, kMaxTaps - 1)] : cur;
+            val[r] = acc;
+            if (c < HD) sq = fmaf(acc, acc, sq);
+            else if (c < HD + GD) sk = fmaf(acc, acc, sk);
+        }
+    }
+    sq = block_allsum(sq, s_red);
+    sk = block_allsum(sk, s_red);
+    const float rq = 1.0f / sqrtf(sq / (float)HD + eps), rk = 1.0f / sqrtf(sk / (float)GD + eps);
+#pragma unroll
+    for (int r = 0; r < kPrepRegs; ++r) {
+        const int c = threadIdx.x + 256 * r;
+        if (c < HD) qout[(size_t)m * ld_q + c] = val[r] * rq * wq[c];
+        else if (c < HD + GD) crow[c - HD] = val[r] * rk * wk[c - HD];
+        else if (c < CC) crow[c - HD] = val[r];
+    }
+}
+
 // Attention without rotation whose q and k are normed over the WHOLE projection (all heads together): one workgroup per row.
 __global__ __launch_bounds__(256) void whole_norm_prep_kernel(float* qkv, int ld, int HD, int GD, int GV, const float* wq, const float* wk, float eps,
                                                               const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
@@ -1134,6 +1208,18 @@ int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, R
     return ZG_OK;
 }
 
+int launch_conv_norm_prep_single(const ConvArgs& a, float* qout, int ld_q, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps,
+                                 const int* row_pos, const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache,
+                                 hipStream_t s, bool* taken) {
+    *taken = false;
+    if (M <= 0 || HD + GD + GV > 256 * kPrepRegs || a.C != HD + GD + GV || a.taps < 1 || a.taps > kMaxTaps || a.bias || a.flags) return ZG_OK;
+    conv_norm_prep_single_kernel<<<M, 256, 0, s>>>(a.in, a.ld_in, qout, ld_q, HD, GD, GV, a.taps, a.w, a.pre_bias, a.tail, a.slot_stride, wq, wk, eps,
+                                                   row_pos, row_slot, page_table, max_pages, page_tokens, cache);
+    ZG_HIP(hipGetLastError());
+    *taken = true;
+    return ZG_OK;
+}
+
 int launch_whole_norm_prep(float* qkv, int ld, int M, int HD, int GD, int GV, const float* wq, const float* wk, float eps, const int* row_pos,
                            const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s) {
     if (M <= 0) return ZG_OK;
@@ -1168,7 +1254,8 @@ size_t window_split_workspace(int rows, int H, int V, int key_capacity, int* n_s
 int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                                   int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
-                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken) {
+                                  size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken,
+                                  const float* out_gate, int ld_gate, float out_factor) {
     *taken = false;
     if (M <= 0) return ZG_OK;
     const int keep = window > 0 ? keep_first : 0;
@@ -1227,7 +1314,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
                                                    key_capacity, st, po);
     }
     ZG_HIP(hipGetLastError());
-    window_merge_kernel<<<M, 256, 0, s>>>(po, n_split, out, ldo, H, V, vfreq, row_pos);
+    window_merge_kernel<<<M, 256, 0, s>>>(po, n_split, out, ldo, H, V, vfreq, row_pos, out_gate, ld_gate, out_factor);
     ZG_HIP(hipGetLastError());
     *taken = true;
     return ZG_OK;
@@ -1285,6 +1372,11 @@ int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const f
                      float factor) {
     const int n_vec = M * rows_per_m;
     if (n_vec <= 0) return ZG_OK;
+    if (width > 256) {  // a workgroup per vector
+        norm_gate_wide_kernel<<<n_vec, 256, 0, s>>>(v, ld, rows_per_m, width, w, eps, gate, ldg, factor);
+        ZG_HIP(hipGetLastError());
+        return ZG_OK;
+    }
     norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg, factor);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
