@@ -921,7 +921,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
                     ZG_TRY(launch_linear(lin, f32, s));
                     lin = Linear();
                     lin.B = L.sdown; lin.ldb = S; lin.C = g->td; lin.ldc = W; lin.M = M; lin.N = W; lin.K = S;
-                    if (few) {  // activation and gate where the second product reads its rows
+                    if (M <= 2) {  // activation and gate where the second product reads its rows (more rows: every workgroup would redo them)
                         lin.A = g->tb; lin.lda = 2 * S + 1; lin.a_glu = S; lin.glu_kind = GLU_CLIPPED; lin.glu_limit = d.shared_limit; lin.glu_gate_col = 2 * S;
                     } else {
                         ZG_TRY(launch_glu_clipped(g->tb, 2 * S + 1, g->tc, M, S, d.shared_limit, nullptr, nullptr, 2 * S, s));

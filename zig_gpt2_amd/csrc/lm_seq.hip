@@ -1090,45 +1090,65 @@ __global__ __launch_bounds__(256) void norm_gate_wide_kernel(float* v, int ld, i
 }
 
 // Decode steps (one row per entry) of the attention below: biases, the short convolutions of q | k | v with their tails moved
-// on, both whole-projection norms, q written normed, keys and values into the cache — one launch; a row's channels (up to
-// 256 * kPrepRegs) stay in registers between the convolution and the norms.
-constexpr int kPrepRegs = 16;
-__global__ __launch_bounds__(256) void conv_norm_prep_single_kernel(const float* in, int ld_in, float* qout, int ld_q, int HD, int GD, int GV, int taps,
-                                                                    const float* cw, const float* pre_bias, float* tail, size_t slot_stride,
-                                                                    const float* wq, const float* wk, float eps, const int* row_pos,
-                                                                    const int* row_slot, const int* page_table, int max_pages, int page_tokens,
-                                                                    float* cache) {
-    __shared__ float s_red[8];
+// on, both whole-projection norms, q written normed, keys and values into the cache — one launch.  A row's channels (up to
+// 256 * kPrepRegs) and their tails (up to kPrepTaps - 1 inputs each) are requested up front and stay in registers; the two
+// statistics share one pair of barriers.
+constexpr int kPrepRegs = 8;
+constexpr int kPrepTaps = 4;
+__global__ __launch_bounds__(256) void conv_norm_prep_single_kernel(const float* __restrict__ in, int ld_in, float* __restrict__ qout, int ld_q, int HD,
+                                                                    int GD, int GV, int taps, const float* __restrict__ cw,
+                                                                    const float* __restrict__ pre_bias, float* __restrict__ tail, size_t slot_stride,
+                                                                    const float* __restrict__ wq, const float* __restrict__ wk, float eps,
+                                                                    const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                                    int page_tokens, float* __restrict__ cache) {
+    __shared__ float s_red[2][4];
     const int m = blockIdx.x, CC = HD + GD + GV, K = taps - 1;
     const int pos = row_pos[m], slot = row_slot[m];
     const int page = page_table[(size_t)slot * max_pages + (pos / page_tokens) % max_pages];
     float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)GD + GV);
     float* tl = tail + (size_t)slot * slot_stride;
+    float cur[kPrepRegs], tv[kPrepRegs][kPrepTaps - 1], wv[kPrepRegs][kPrepTaps];
+#pragma unroll
+    for (int r = 0; r < kPrepRegs; ++r) {
+        const int c = threadIdx.x + 256 * r;
+        const bool ok = c < CC;
+        cur[r] = ok ? in[(size_t)m * ld_in + c] + (pre_bias ? pre_bias[c] : 0.0f) : 0.0f;
+#pragma unroll
+        for (int j = 0; j < kPrepTaps - 1; ++j) tv[r][j] = (ok && j < K) ? tl[(size_t)j * CC + c] : 0.0f;
+#pragma unroll
+        for (int j = 0; j < kPrepTaps; ++j) wv[r][j] = (ok && j < taps) ? cw[(size_t)c * taps + j] : 0.0f;
+    }
     float val[kPrepRegs];
     float sq = 0.0f, sk = 0.0f;
 #pragma unroll
     for (int r = 0; r < kPrepRegs; ++r) {
         const int c = threadIdx.x + 256 * r;
-        val[r] = 0.0f;
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < kPrepTaps; ++j) {  // tap j < K reads the tail's input j (oldest first), tap K the current one
+            float xin = cur[r];
+#pragma unroll
+            for (int u = 0; u < kPrepTaps - 1; ++u) xin = (j < K && u == j) ? tv[r][u] : xin;
+            if (j <= K) acc = fmaf(wv[r][j], xin, acc);
+        }
+        val[r] = acc;
+        if (c < HD) sq = fmaf(acc, acc, sq);
+        else if (c < HD + GD) sk = fmaf(acc, acc, sk);
         if (c < CC) {
-            const float cur = in[(size_t)m * ld_in + c] + (pre_bias ? pre_bias[c] : 0.0f);
-            float tv[kMaxTaps];
 #pragma unroll
-            for (int j = 0; j < kMaxTaps; ++j) tv[j] = j < K ? tl[(size_t)j * CC + c] : 0.0f;
-            float acc = cw[(size_t)c * taps + K] * cur;
-#pragma unroll
-            for (int j = 0; j < kMaxTaps; ++j)
-                if (j < K) acc = fmaf(cw[(size_t)c * taps + j], tv[j], acc);
-#pragma unroll
-            for (int j = 0; j < kMaxTaps; ++j)
-                if (j < K) tl[(size_t)j * CC + c] = j + 1 < K ? tv[min(j + 1, kMaxTaps - 1)] : cur;
-            val[r] = acc;
-            if (c < HD) sq = fmaf(acc, acc, sq);
-            else if (c < HD + GD) sk = fmaf(acc, acc, sk);
+            for (int j = 0; j < kPrepTaps - 1; ++j)
+                if (j < K) tl[(size_t)j * CC + c] = (j + 1 < K && j + 1 < kPrepTaps - 1) ? tv[r][(j + 1) % (kPrepTaps - 1)] : cur[r];
         }
     }
-    sq = block_allsum(sq, s_red);
-    sk = block_allsum(sk, s_red);
+    sq = wave_allsum(sq);
+    sk = wave_allsum(sk);
+    if ((threadIdx.x & 63) == 0) {
+        s_red[0][threadIdx.x >> 6] = sq;
+        s_red[1][threadIdx.x >> 6] = sk;
+    }
+    __syncthreads();
+    sq = (s_red[0][0] + s_red[0][1]) + (s_red[0][2] + s_red[0][3]);
+    sk = (s_red[1][0] + s_red[1][1]) + (s_red[1][2] + s_red[1][3]);
     const float rq = 1.0f / sqrtf(sq / (float)HD + eps), rk = 1.0f / sqrtf(sk / (float)GD + eps);
 #pragma unroll
     for (int r = 0; r < kPrepRegs; ++r) {
@@ -1212,7 +1232,7 @@ int launch_conv_norm_prep_single(const ConvArgs& a, float* qout, int ld_q, int M
                                  const int* row_pos, const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache,
                                  hipStream_t s, bool* taken) {
     *taken = false;
-    if (M <= 0 || HD + GD + GV > 256 * kPrepRegs || a.C != HD + GD + GV || a.taps < 1 || a.taps > kMaxTaps || a.bias || a.flags) return ZG_OK;
+    if (M <= 0 || HD + GD + GV > 256 * kPrepRegs || a.C != HD + GD + GV || a.taps < 1 || a.taps > kPrepTaps || a.bias || a.flags) return ZG_OK;
     conv_norm_prep_single_kernel<<<M, 256, 0, s>>>(a.in, a.ld_in, qout, ld_q, HD, GD, GV, a.taps, a.w, a.pre_bias, a.tail, a.slot_stride, wq, wk, eps,
                                                    row_pos, row_slot, page_table, max_pages, page_tokens, cache);
     ZG_HIP(hipGetLastError());
