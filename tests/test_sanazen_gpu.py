@@ -447,3 +447,41 @@ def test_errors_are_reported():
     with pytest.raises(ValueError):
         lm.LMConfig.from_json(bad)
     m.close()
+
+
+def _random_cfg(rng):
+    """A stack with sizes drawn at random: odd and even widths, heads on fewer key heads, unequal key and value sizes, windows
+    from one token to none, kept tokens below and above the window, 0 to 6 taps, experts with and without a shared one."""
+    layers = []
+    for _ in range(int(rng.integers(1, 4))):
+        kv = int(rng.choice([1, 2, 3]))
+        heads = kv * int(rng.choice([1, 2, 4]))
+        window = int(rng.choice([0, 1, 2, 5, 16, 33, 64, 100]))
+        lh = int(rng.integers(1, 4))
+        mlp = None
+        if rng.random() < 0.75:
+            experts = int(rng.integers(1, 10))
+            mlp = sl.moe_mlp(ff=int(rng.integers(1, 40)), experts=experts, top=int(rng.integers(1, experts + 1)), limit=float(rng.choice([0.25, 1.0, 7.0])),
+                             shared=(int(rng.integers(1, 40)), float(rng.choice([0.5, 3.0]))) if rng.random() < 0.6 else None)
+        layers.append(sl.pair_layer(heads=heads, kv_heads=kv, dim=int(rng.integers(1, 40)), vdim=int(rng.integers(1, 40)), window=window,
+                                    keep_first=int(rng.choice([0, 1, 3, 8, 40])), scale=float(rng.choice([0.1, 0.5])), conv=int(rng.integers(0, 7)),
+                                    lin_heads=lh, lin_dim=int(rng.integers(1, 50)), lin_vdim=int(rng.integers(1, 50)),
+                                    decay=[float(v) for v in rng.uniform(0.3, 1.0, lh)], left_scale=float(rng.uniform(0.3, 1.5)),
+                                    right_scale=float(rng.uniform(0.3, 1.5)), mlp=mlp))
+    return sl.config(layers, vocab=int(rng.integers(2, 300)), width=int(rng.integers(3, 90)), eps=float(rng.choice([1e-6, 1e-5, 1e-3])),
+                     embed_scale=float(rng.uniform(0.5, 9.0)), logit_scale=float(rng.uniform(0.2, 2.0)), softcap=float(rng.choice([0.0, 5.0, 40.0])))
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_sizes_drawn_at_random(seed):
+    rng = np.random.default_rng(7000 + seed)
+    cfg = _random_cfg(rng)
+    w = sl.weights(cfg, seed=seed)
+    n = int(rng.integers(20, 300))
+    toks = sl.tokens(seed, n, cfg["vocab"])
+    ref = so.forward(w, cfg, toks)[0]
+    m = make(cfg, w, page_tokens=int(rng.choice([4, 16, 64])))
+    tl.assert_close(run_whole(m, toks), ref, "float32", cfg)
+    cuts = sorted(set(int(c) for c in rng.integers(1, n, 6))) + list(range(max(1, n - 12), n))
+    tl.assert_close(run_cut(m, toks, sorted(set(cuts))), ref, "float32", (cfg, cuts))
+    m.close()
