@@ -278,9 +278,13 @@ def test_far_keys_among_hundreds():
     m.close()
 
 
-def test_linear_attention_remembers_far_tokens():
+@pytest.mark.parametrize("scan", [False, True])
+def test_linear_attention_remembers_far_tokens(monkeypatch, scan):
     """Decays close to one: the state forgets slowly, so the first tokens still weigh in hundreds of tokens later (far beyond
-    the window) — a state that is lost, reset or carried wrongly between portions, chunks or steps shows."""
+    the window) — a state that is lost, reset or carried wrongly between portions, chunks or steps shows.  Prompt portions take
+    chunks of 32 tokens as matrix products; the hook sends them through the token-serial scan (what wider heads take)."""
+    if scan:
+        monkeypatch.setenv("ZGPT2_LM_LINEAR_NO_CHUNKS", "1")
     cfg = sl.config([sl.pair_layer(window=5, keep_first=0, lin_heads=2, lin_dim=16, lin_vdim=12, decay=[0.9995, 0.998], left_scale=0.3, right_scale=1.0)], width=32)
     w = sl.weights(cfg, seed=11)
     n = 600
@@ -291,7 +295,7 @@ def test_linear_attention_remembers_far_tokens():
     assert tl.rel_err(ref_other[-1], ref[-1]) > 1e-3, "the construction does not carry the first tokens to the end"
     m = make(cfg, w, max_tokens=1024)
     tl.assert_close(run_whole(m, toks), ref, "float32")  # long enough for the chunks that run side by side
-    tl.assert_close(run_cut(m, toks, [2, 4, 100, 101, 103, 200, 500]), ref, "float32")
+    tl.assert_close(run_cut(m, toks, [2, 4, 100, 101, 103, 200, 231, 232, 233, 264, 500]), ref, "float32")
     tl.assert_close(run_cut(m, toks, [300] + list(range(540, n))), ref, "float32")
     m.close()
 

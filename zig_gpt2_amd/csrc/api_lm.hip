@@ -547,7 +547,7 @@ void layout(zg_lm* g, Bump& b) {
     g->sorted = b.take<int>(MS * max_assign);
     g->inv = b.take<int>(MS * max_assign);
     g->grp_off = b.take<int>(max_e + 1);
-    g->scan_ws_floats = (MS / 64 + 1 + NS) * max_scan;
+    g->scan_ws_floats = (MS / 32 + 1 + NS) * max_scan;  // a state per chunk of the chunked recurrences (chunks of 64 or 32 tokens)
     g->scan_ws = b.take<float>(std::max<size_t>(1, g->scan_ws_floats));
     g->attn_ws_floats = (size_t)kGemvMaxRows * kAttnSplits * max_att_part;
     g->attn_ws = b.take<float>(std::max<size_t>(1, g->attn_ws_floats));

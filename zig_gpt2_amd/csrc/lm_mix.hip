@@ -2,6 +2,7 @@
 // the residual sum fused in), the gated linear recurrence (HGRN2) and the latent attention over a paged cache of latents.
 // Everything here is fp32 in both precision modes: norms, gates, the recurrent state, positions, angles, scores and weights.
 #include <math.h>
+#include <stdlib.h>
 
 #include <algorithm>
 
@@ -472,13 +473,13 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
 
 // phase B: one thread per state element walks the chunks of its entry
 __global__ __launch_bounds__(256) void hgrn2_carry_kernel(float* state, size_t slot_stride, const int* ent_len, const int* ent_slot, int n_entries, int H,
-                                                          int D, int V, float* wsB, const float* wsA) {
+                                                          int D, int V, float* wsB, const float* wsA, int chunk) {
     const int e = blockIdx.y;
     const size_t n = (size_t)H * D * V, idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= n) return;
     int first = 0;
-    for (int k = 0; k < e; ++k) first += (ent_len[k] + kScanChunk - 1) / kScanChunk;
-    const int nc = (ent_len[e] + kScanChunk - 1) / kScanChunk;
+    for (int k = 0; k < e; ++k) first += (ent_len[k] + chunk - 1) / chunk;
+    const int nc = (ent_len[e] + chunk - 1) / chunk;
     const size_t hi = idx / V;  // (head, row)
     float* slot = state + (size_t)ent_slot[e] * slot_stride;
     float S = slot[idx];
@@ -489,6 +490,143 @@ __global__ __launch_bounds__(256) void hgrn2_carry_kernel(float* state, size_t s
         S = fmaf(A, S, B);
     }
     if (nc > 0) slot[idx] = S;
+}
+
+// ------------------------------------------------------------------------------------------------ linear attention, chunks on the matrix cores
+// With ONE decay per head the recurrence S <- lambda S + k v^T, o = S^T q of a chunk of n <= 32 tokens is three matrix products
+// (true fp32, v_mfma_f32_32x32x2_f32; q, k, v through silu on load):
+//   state   B = sum_j lambda^(n-1-j) k_j v_j^T                       the chunk's end state from zero          (phase A, per chunk)
+//   carry   S_start(c + 1) = lambda^n S_start(c) + B_c               down the chunks of an entry              (hgrn2_carry_kernel)
+//   output  o_i = sum_(j<=i) lambda^(i-j) (q_i . k_j) v_j + lambda^(i+1) S_start^T q_i                        (phase C, per chunk)
+// A workgroup takes a (chunk, head); lane (r, half) of a wave holds channels half * Dh .. of row r (the order inside a dot product
+// is free), tokens half * 16 .. where the tokens are the product's inner dimension.
+constexpr int kLinChunk = 32;
+typedef __attribute__((ext_vector_type(16))) float f32x16_lin;
+
+__device__ __forceinline__ float decay_pow(float lam, float l2, int n) { return n <= 0 ? 1.0f : (lam <= 0.0f ? 0.0f : exp2f((float)n * l2)); }
+
+__device__ __forceinline__ bool lin_find_chunk(int id, const int* ent_len, int n_entries, int& e, int& c) {
+    for (e = 0; e < n_entries; ++e) {
+        const int nc = (ent_len[e] + kLinChunk - 1) / kLinChunk;
+        if (id < nc) {
+            c = id;
+            return true;
+        }
+        id -= nc;
+    }
+    return false;
+}
+
+__global__ __launch_bounds__(256) void linear_chunk_state_kernel(const float* __restrict__ proj, int ld, const int* ent_start, const int* ent_len,
+                                                                 int n_entries, int H, int D, int V, const float* decay, float* __restrict__ wsB,
+                                                                 float* __restrict__ wsA) {
+    int e, c;
+    if (!lin_find_chunk(blockIdx.x, ent_len, n_entries, e, c)) return;
+    const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, kh = lane >> 5;
+    const int n = min(kLinChunk, ent_len[e] - c * kLinChunk), m0 = ent_start[e] + c * kLinChunk, HD = H * D;
+    const float lam = decay[h], l2 = lam > 0.0f ? log2f(lam) : 0.0f;
+    const float* kbase = proj + (size_t)m0 * ld + HD + (size_t)h * D;
+    const float* vbase = proj + (size_t)m0 * ld + 2 * HD + (size_t)h * V;
+    float* B = wsB + ((size_t)blockIdx.x * H + h) * D * V;
+    const int tilesD = (D + 31) / 32, tilesV = (V + 31) / 32;
+    for (int tile = wave; tile < tilesD * tilesV; tile += 4) {
+        const int d0 = (tile / tilesV) * 32, v0 = (tile % tilesV) * 32;
+        float a[16], b[16];
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {  // token j is the inner dimension: weight lambda^(n - 1 - j) on the key
+            const int j = kh * 16 + t;
+            a[t] = (j < n && d0 + r < D) ? kbase[(size_t)j * ld + d0 + r] : 0.0f;
+            b[t] = (j < n && v0 + r < V) ? vbase[(size_t)j * ld + v0 + r] : 0.0f;
+        }
+        f32x16_lin acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 16; ++t)
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(silu_f(a[t]) * decay_pow(lam, l2, n - 1 - (kh * 16 + t)), silu_f(b[t]), acc, 0, 0, 0);
+        // accumulator element i: row 8 (i / 4) + 4 half + i % 4, column r
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int d = d0 + 8 * (i >> 2) + 4 * kh + (i & 3);
+            if (d < D && v0 + r < V) B[(size_t)d * V + v0 + r] = acc[i];
+        }
+    }
+    for (int i = threadIdx.x; i < D; i += blockDim.x) wsA[((size_t)blockIdx.x * H + h) * D + i] = decay_pow(lam, l2, n);
+}
+
+template <int DH>
+__global__ __launch_bounds__(256) void linear_chunk_out_kernel(const float* __restrict__ proj, int ld, float* __restrict__ out, int ldo,
+                                                               const int* ent_start, const int* ent_len, int n_entries, int H, int D, int V,
+                                                               const float* decay, const float* __restrict__ wsB) {
+    __shared__ float s_p[4][32][33];
+    int e, c;
+    if (!lin_find_chunk(blockIdx.x, ent_len, n_entries, e, c)) return;
+    const int h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, kh = lane >> 5;
+    const int n = min(kLinChunk, ent_len[e] - c * kLinChunk), m0 = ent_start[e] + c * kLinChunk, HD = H * D, Dh = (D + 1) / 2;
+    const float lam = decay[h], l2 = lam > 0.0f ? log2f(lam) : 0.0f;
+    const float* S = wsB + ((size_t)blockIdx.x * H + h) * D * V;  // the chunk's start state (the carry left it here)
+    const float* qrow = proj + (size_t)(m0 + min(r, n - 1)) * ld + (size_t)h * D + kh * Dh;
+    const float* krow = qrow + HD;
+    const float* vbase = proj + (size_t)m0 * ld + 2 * HD + (size_t)h * V;
+    float qreg[DH], kreg[DH];
+#pragma unroll
+    for (int t = 0; t < DH; ++t) {
+        const bool ok = r < n && t < Dh && kh * Dh + t < D;
+        qreg[t] = ok ? qrow[t] : 0.0f;
+        kreg[t] = ok ? krow[t] : 0.0f;
+    }
+#pragma unroll
+    for (int t = 0; t < DH; ++t) {
+        qreg[t] = silu_f(qreg[t]);
+        kreg[t] = silu_f(kreg[t]);
+    }
+    f32x16_lin acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int t = 0; t < DH; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[t], kreg[t], acc, 0, 0, 0);
+    // element i: query 8 (i / 4) + 4 half + i % 4, key r: the decay of their distance, nothing for keys behind the query
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const int qi = 8 * (i >> 2) + 4 * kh + (i & 3);
+        s_p[wave][qi][r] = (r <= qi && qi < n) ? acc[i] * decay_pow(lam, l2, qi - r) : 0.0f;
+    }
+    __syncthreads();
+    const float carry = decay_pow(lam, l2, r + 1);  // what the start state has decayed to when token r reads it
+#pragma unroll
+    for (int t = 0; t < DH; ++t) qreg[t] *= carry;
+    const int tilesV = (V + 31) / 32;
+    for (int vt = wave; vt < tilesV; vt += 4) {
+        const int v0 = vt * 32;
+        const bool col_ok = v0 + r < V;
+        float vv[16];
+#pragma unroll
+        for (int t = 0; t < 16; ++t) {
+            const int j = kh * 16 + t;
+            vv[t] = (j < n && col_ok) ? vbase[(size_t)j * ld + v0 + r] : 0.0f;
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.0f;
+#pragma unroll
+        for (int t = 0; t < 16; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(s_p[wave][r][kh * 16 + t], silu_f(vv[t]), acc, 0, 0, 0);
+#pragma unroll
+        for (int t0 = 0; t0 < DH; t0 += 16) {  // the start state's share, 16 state rows requested at a time
+            float sv[16];
+#pragma unroll
+            for (int u = 0; u < 16; ++u) {
+                const int t = t0 + u, ch = kh * Dh + t;
+                sv[u] = (t < DH && t < Dh && ch < D && col_ok) ? S[(size_t)ch * V + v0 + r] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 16; ++u)
+                if (t0 + u < DH) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qreg[min(t0 + u, DH - 1)], sv[u], acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int qi = 8 * (i >> 2) + 4 * kh + (i & 3);
+            if (qi < n && col_ok) out[(size_t)(m0 + qi) * ldo + (size_t)h * V + v0 + r] = acc[i];
+        }
+    }
 }
 
 // ------------------------------------------------------------------------------------------------ latent attention
@@ -989,6 +1127,28 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
                       float* ws, size_t ws_floats, hipStream_t s, const float* decay) {
     if (n_entries <= 0) return ZG_OK;
     ZG_REQUIRE(D >= 1 && D <= 16 * kScanRows, ZG_ERR_UNSUPPORTED, "hgrn2: %d key channels per head (at most %d)", D, 16 * kScanRows);
+    if (decay && M > kGemvMaxRows && D <= 128 && ws && getenv("ZGPT2_LM_LINEAR_NO_CHUNKS") == nullptr) {
+        // a scalar decay per head: chunks of kLinChunk tokens as matrix products (prompt portions; the test hook sends them through the scan)
+        const int n_chunks = (M + kLinChunk - 1) / kLinChunk + n_entries;
+        const size_t hf = (size_t)H * D * V;
+        if (ws_floats >= (size_t)n_chunks * (hf + (size_t)H * D) && n_chunks <= 65535 && H <= 65535) {
+            float* cB = ws;
+            float* cA = ws + (size_t)n_chunks * hf;
+            const dim3 grid(n_chunks, H);
+            linear_chunk_state_kernel<<<grid, 256, 0, s>>>(proj, ld, ent_start, ent_len, n_entries, H, D, V, decay, cB, cA);
+            ZG_HIP(hipGetLastError());
+            hgrn2_carry_kernel<<<dim3((unsigned)((hf + 255) / 256), n_entries), 256, 0, s>>>(state, slot_stride, ent_len, ent_slot, n_entries, H, D, V, cB,
+                                                                                          cA, kLinChunk);
+            ZG_HIP(hipGetLastError());
+            const int dh = (D + 1) / 2;
+            if (dh <= 8) linear_chunk_out_kernel<8><<<grid, 256, 0, s>>>(proj, ld, out, ldo, ent_start, ent_len, n_entries, H, D, V, decay, cB);
+            else if (dh <= 16) linear_chunk_out_kernel<16><<<grid, 256, 0, s>>>(proj, ld, out, ldo, ent_start, ent_len, n_entries, H, D, V, decay, cB);
+            else if (dh <= 32) linear_chunk_out_kernel<32><<<grid, 256, 0, s>>>(proj, ld, out, ldo, ent_start, ent_len, n_entries, H, D, V, decay, cB);
+            else linear_chunk_out_kernel<64><<<grid, 256, 0, s>>>(proj, ld, out, ldo, ent_start, ent_len, n_entries, H, D, V, decay, cB);
+            ZG_HIP(hipGetLastError());
+            return ZG_OK;
+        }
+    }
     int G = 1;
     while (G * kScanRows < D) G <<= 1;
     const int Dp = G * kScanRows;
@@ -1028,7 +1188,7 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
     ZG_SCAN_G(max_chunks, SCAN_A);
     ZG_HIP(hipGetLastError());
     hgrn2_carry_kernel<<<dim3((unsigned)((head_floats + 255) / 256), n_entries), 256, 0, s>>>(state, slot_stride, ent_len, ent_slot, n_entries, H, D, V,
-                                                                                                wsB, wsA);
+                                                                                                wsB, wsA, kScanChunk);
     ZG_HIP(hipGetLastError());
     ZG_SCAN_G(max_chunks, SCAN_C);
     ZG_HIP(hipGetLastError());
