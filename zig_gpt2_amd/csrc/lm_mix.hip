@@ -483,11 +483,20 @@ __global__ __launch_bounds__(256) void hgrn2_carry_kernel(float* state, size_t s
     const size_t hi = idx / V;  // (head, row)
     float* slot = state + (size_t)ent_slot[e] * slot_stride;
     float S = slot[idx];
-    for (int c = 0; c < nc; ++c) {
-        float* b = wsB + (size_t)(first + c) * n + idx;
-        const float B = *b, A = wsA[(size_t)(first + c) * H * D + hi];
-        *b = S;  // the chunk's start state for phase C
-        S = fmaf(A, S, B);
+    for (int c0 = 0; c0 < nc; c0 += 8) {  // eight chunks' operands requested together: the chain itself is eight multiply-adds
+        float Bv[8], Av[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int c = min(c0 + u, nc - 1);
+            Bv[u] = wsB[(size_t)(first + c) * n + idx];
+            Av[u] = wsA[(size_t)(first + c) * H * D + hi];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (c0 + u < nc) {
+                wsB[(size_t)(first + c0 + u) * n + idx] = S;  // the chunk's start state for phase C
+                S = fmaf(Av[u], S, Bv[u]);
+            }
     }
     if (nc > 0) slot[idx] = S;
 }
@@ -529,7 +538,7 @@ __global__ __launch_bounds__(256) void linear_chunk_state_kernel(const float* __
     const float* vbase = proj + (size_t)m0 * ld + 2 * HD + (size_t)h * V;
     float* B = wsB + ((size_t)blockIdx.x * H + h) * D * V;
     const int tilesD = (D + 31) / 32, tilesV = (V + 31) / 32;
-    for (int tile = wave; tile < tilesD * tilesV; tile += 4) {
+    for (int tile = blockIdx.z * 4 + wave; tile < tilesD * tilesV; tile += 4 * gridDim.z) {
         const int d0 = (tile / tilesV) * 32, v0 = (tile % tilesV) * 32;
         float a[16], b[16];
 #pragma unroll
@@ -551,7 +560,8 @@ __global__ __launch_bounds__(256) void linear_chunk_state_kernel(const float* __
             if (d < D && v0 + r < V) B[(size_t)d * V + v0 + r] = acc[i];
         }
     }
-    for (int i = threadIdx.x; i < D; i += blockDim.x) wsA[((size_t)blockIdx.x * H + h) * D + i] = decay_pow(lam, l2, n);
+    if (blockIdx.z == 0)
+        for (int i = threadIdx.x; i < D; i += blockDim.x) wsA[((size_t)blockIdx.x * H + h) * D + i] = decay_pow(lam, l2, n);
 }
 
 template <int DH>
@@ -569,11 +579,24 @@ __global__ __launch_bounds__(256) void linear_chunk_out_kernel(const float* __re
     const float* krow = qrow + HD;
     const float* vbase = proj + (size_t)m0 * ld + 2 * HD + (size_t)h * V;
     float qreg[DH], kreg[DH];
+    // 16-byte loads where a lane's run of channels starts on a 16-byte boundary and is a multiple of four long
+    const bool vec = D % 8 == 0 && ld % 4 == 0 && (reinterpret_cast<uintptr_t>(proj) & 15) == 0;
+    if (vec) {
 #pragma unroll
-    for (int t = 0; t < DH; ++t) {
-        const bool ok = r < n && t < Dh && kh * Dh + t < D;
-        qreg[t] = ok ? qrow[t] : 0.0f;
-        kreg[t] = ok ? krow[t] : 0.0f;
+        for (int t = 0; t < DH; t += 4) {
+            const bool ok = r < n && t < Dh;
+            const f32x4 a = ok ? *reinterpret_cast<const f32x4*>(qrow + t) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            const f32x4 b = ok ? *reinterpret_cast<const f32x4*>(krow + t) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            qreg[t] = a.x; qreg[t + 1] = a.y; qreg[t + 2] = a.z; qreg[t + 3] = a.w;
+            kreg[t] = b.x; kreg[t + 1] = b.y; kreg[t + 2] = b.z; kreg[t + 3] = b.w;
+        }
+    } else {
+#pragma unroll
+        for (int t = 0; t < DH; ++t) {
+            const bool ok = r < n && t < Dh && kh * Dh + t < D;
+            qreg[t] = ok ? qrow[t] : 0.0f;
+            kreg[t] = ok ? krow[t] : 0.0f;
+        }
     }
 #pragma unroll
     for (int t = 0; t < DH; ++t) {
@@ -1135,7 +1158,8 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
             float* cB = ws;
             float* cA = ws + (size_t)n_chunks * hf;
             const dim3 grid(n_chunks, H);
-            linear_chunk_state_kernel<<<grid, 256, 0, s>>>(proj, ld, ent_start, ent_len, n_entries, H, D, V, decay, cB, cA);
+            const int tiles = ((D + 31) / 32) * ((V + 31) / 32);
+            linear_chunk_state_kernel<<<dim3(n_chunks, H, std::min(16, (tiles + 3) / 4)), 256, 0, s>>>(proj, ld, ent_start, ent_len, n_entries, H, D, V, decay, cB, cA);
             ZG_HIP(hipGetLastError());
             hgrn2_carry_kernel<<<dim3((unsigned)((hf + 255) / 256), n_entries), 256, 0, s>>>(state, slot_stride, ent_len, ent_slot, n_entries, H, D, V, cB,
                                                                                           cA, kLinChunk);
