@@ -364,13 +364,22 @@ enum {
     ZG_LM_MIX_CHANNEL_DELTA = 4,    /* gated delta rule with a decay per key channel: S = diag(g) S; u = beta (v - S^T k);
                                        S += k u^T; o = S^T q;  q, k, v behind short causal convolutions + silu, q and k of unit
                                        length, the decay and the output gate through two-step (low-rank) projections */
-    ZG_LM_MIX_WINDOW_LINEAR = 5     /* two branches on the same input, c_left * left + c_right * right:
+    ZG_LM_MIX_WINDOW_LINEAR = 5,    /* two branches on the same input, c_left * left + c_right * right:
                                        left   grouped-query softmax attention (no rotation) whose q, k, v = conv(W h + b) pass a short
                                               causal convolution and whose q and k are RMS-normed over the WHOLE projection; a query sees
                                               the keys inside its window and, beyond it, the first keep_first tokens of the sequence;
                                               the heads are gated by sigmoid(W_g h), the output projection has a bias;
                                        right  linear attention with one fixed decay per head: q, k, v = silu(W h), S = decay_h S + k v^T,
                                               o = S^T q; the heads RMS-normed together, gated by sigmoid(W_g h) */
+    ZG_LM_MIX_GLA = 6,              /* gated linear attention with a decay per key channel: q = W_q h / sqrt(dim), k, v, gate plain
+                                       projections; f = sigmoid(W_a2 W_a1 h + b_a)^(1 / tau);  S = diag(f) S + k v^T;  o = S^T q;
+                                       every head's o RMS-normed over vdim with one plain weight [vdim], times silu(W_g h), then W_o */
+    ZG_LM_MIX_ATTENTION = 7         /* causal grouped-query softmax attention over the whole sequence, no rotation, no value
+                                       projection: the VALUE of a key head is that head's un-normalised key; q and k are divided by their
+                                       root mean square per head (no weight); the query of position p is multiplied by
+                                       1 + qtemp_coef ln(floor((p + 1) / qtemp_every) + 1) (qtemp_every 0: not);
+                                       score = scale q . k, then softcap tanh(score / softcap) (softcap 0: not), then minus
+                                       2^(-8 (h + 1) / heads) (i - j) for head h (dist_bias 0: not) */
 };
 enum { ZG_LM_FF_NONE = 0, ZG_LM_FF_DENSE = 1 /* down(relu(up h)^2) */, ZG_LM_FF_MOE = 2 /* top-k of `experts` units */ };
 /* Activation of an expert (ff_act) and the rule of the router (router) of ZG_LM_FF_MOE. */
@@ -382,8 +391,12 @@ enum {
 enum {
     ZG_LM_ROUTE_SOFTMAX_ALL = 0, /* s = softmax over all experts; the `top` largest s + correction; weights s */
     ZG_LM_ROUTE_TOP_LOGITS = 1,  /* z = router h + bias (`router.b`); the `top` largest z; weights softmax over the chosen z */
-    ZG_LM_ROUTE_SIGMOID_INPUT = 2 /* s = sigmoid(router h); the `top` largest; the weight s (not renormalised) multiplies the expert's
+    ZG_LM_ROUTE_SIGMOID_INPUT = 2, /* s = sigmoid(router h); the `top` largest; the weight s (not renormalised) multiplies the expert's
                                      INPUT: the sublayer's output is the plain sum of expert(s h) */
+    ZG_LM_ROUTE_SIGMOID_GROUPS = 3 /* s = sigmoid(router h); experts are ranked by r = s + correction.  The expert list is cut into
+                                     route_groups contiguous blocks of equal size; a block's rank is r of its best expert plus r of
+                                     its second best (a block of one: its only r); experts outside the route_keep top-ranked blocks
+                                     get r = -inf; the `top` highest r win; weights s / (sum of the winners' s + 1e-20) * route_scale */
 };
 enum { ZG_LM_ROT_PLAIN = 0, ZG_LM_ROT_YARN = 1 /* blend by pair index, amplitude factor */, ZG_LM_ROT_BANDS = 2 /* by wavelength: see rot_* */ };
 typedef struct {
@@ -411,9 +424,20 @@ typedef struct {
     int lin_heads, lin_dim, lin_vdim; /* window + linear pair: heads, key and value channels per head of the linear-attention branch
                                          (its decays: the fp32 tensor `mix.right.decay` [lin_heads], which the host fills from config.json) */
     float ff_limit;               /* ZG_LM_ACT_GLU_CLIPPED: the experts' clip */
-    int shared_width;             /* > 0: a shared expert of this hidden width (same activation) runs for every token and is added,
-                                     times sigmoid(shared.sg . h) (tensors shared.gate / up / down / sg) */
+    int shared_width;             /* > 0: a shared expert of this hidden width (same activation) runs for every token and is added;
+                                     with the clipped activation times sigmoid(shared.sg . h) (tensors shared.gate / up / down / sg),
+                                     with ZG_LM_ACT_GLU_SILU as it is (tensors shared.gate / up / down) */
     float shared_limit;           /* its clip */
+    /* (the fields below are zero for the designs that do not name them) */
+    float tau;                    /* gated linear attention: the decay is sigmoid(.)^(1 / tau) */
+    float softcap;                /* attention: > 0: score <- softcap tanh(score / softcap) */
+    float qtemp_coef;             /* attention: query factor 1 + qtemp_coef ln(floor((p + 1) / qtemp_every) + 1) ... */
+    int qtemp_every;              /* ... 0: no such factor */
+    int dist_bias;                /* attention: != 0: head h's scores lose 2^(-8 (h + 1) / heads) per position of distance */
+    int route_groups, route_keep; /* ZG_LM_ROUTE_SIGMOID_GROUPS: contiguous blocks of experts (0: one), and how many of them stay (0: all) */
+    float route_scale;            /* ZG_LM_ROUTE_SIGMOID_GROUPS: factor of the normalised weights (0: 1) */
+    int weights_of;               /* > 0: this layer owns no tensors and runs those of layer weights_of - 1 (whose other fields it
+                                     repeats) with separate cache and state */
 } zg_lm_layer;
 enum {
     ZG_LM_F32 = 1 << 0,     /* true 32-bit products everywhere */
@@ -423,13 +447,18 @@ enum {
     ZG_LM_SIDE_BY_SIDE = 1 << 4, /* a layer is x += mixer(norm1(x)) + ff(norm2(x)), both sublayers reading the same x; norm weights are
                                     plain factors (not offsets from one), no norm behind a sublayer (no norm1b / norm2b), no token
                                     shift; `final.norm` is a plain factor too */
-    ZG_LM_SINUSOID_POSITIONS = 1 << 5 /* the embedding output gets the position's vector added: entry 2i = sin(p 10000^(-2i/width)),
+    ZG_LM_SINUSOID_POSITIONS = 1 << 5, /* the embedding output gets the position's vector added: entry 2i = sin(p 10000^(-2i/width)),
                                          entry 2i + 1 = cos of the same angle (fp32 position x fp32 frequency) */
+    ZG_LM_TANH_NORMS = 1 << 6, /* every norm of the stack (norm1, norm1b, norm2, norm2b, final.norm) is tanh(alpha v) * w + b — elementwise, nothing
+                                  is reduced over the row — with the scalar `<name>.alpha` and the vector `<name>.b` beside the weight `<name>`; the
+                                  mixer reads norm1(x) as it is (no token shift, no input convolution), and a sublayer's normed output
+                                  enters the residual sum times residual_mult */
+    ZG_LM_EMBED_NORM = 1 << 7  /* the embedding output passes the stack's norm with the tensors `embed.norm` (ZG_LM_TANH_NORMS only) */
 };
 typedef struct {
     size_t vocab, width, n_layers;
     const zg_lm_layer* layers;
-    int loop_start, loop_stop, loop_times; /* layers [start, stop) run `times` times in a row, every pass with a state of its own; times <= 1: no loop */
+    int loop_start, loop_stop, loop_times; /* layers [start, stop) run `times` times in a row, every pass with separate state; times <= 1: no loop */
     float norm_eps;
     size_t max_tokens;      /* tokens that all open sequences may hold together (sizes the latent cache) */
     size_t max_seqs;        /* state slots */
@@ -442,17 +471,19 @@ typedef struct {
                                `canon2` [width][taps], last column = the current token); a slot keeps the taps - 1 last inputs */
     float logit_scale;      /* logits = head . norm(x) * logit_scale (0: 1) */
     float logit_softcap;    /* > 0: logits <- cap tanh(logits / cap) */
+    float residual_mult;    /* ZG_LM_TANH_NORMS: x += residual_mult * norm(sublayer output) (0: 1) */
 } zg_lm_config;
 typedef struct zg_lm zg_lm;
 /* One arena for weights, state and scratch; the handle owns a stream on `device`.  Needs no zg_init. */
 int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device);
 int zg_lm_destroy(zg_lm* g);
-/* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift|canon1|canon2`,
+/* Weights by checkpoint name: `embed`, `head`, `final.norm`, and per layer i `l<i>.norm1|norm1b|norm2|norm2b|shift|canon1|canon2`
+ * (ZG_LM_TANH_NORMS: each norm also `.b` and `.alpha`; `embed.norm` likewise),
  * `l<i>.mix.*` (hgrn2: q f f.b lower v norm o; latent attention: dq dq.norm uq dkv dkv.norm uk uv o; parallel: left.q left.k
  * left.v left.sink left.talk left.o left.out right.y right.y.b right.x right.x.b right.conv right.conv.b right.ra right.ra.b
  * right.ri right.ri.b right.lam right.o right.out; delta rule: q q.conv k k.conv v v.conv b A_log dt_bias a1 a2 g1 g2 norm o;
  * window + linear pair: left.q|k|v with .b and .conv each, left.q.norm left.k.norm left.g left.o left.o.b right.q right.k right.v
- * right.g right.norm right.o right.decay)
+ * right.g right.norm right.o right.decay; gated linear attention: q k v g o norm a1 a2 a2.b; attention: q k o)
  * and `l<i>.mlp.*` (dense: up down; experts: e<j>.gate e<j>.up e<j>.down router, and correction or router.b; shared.gate shared.up
  * shared.down shared.sg).  data: fp32 on the host, `len` elements, matrices
  * [out][in] row-major; matrices are stored bf16 (round to nearest even).  ZG_ERR_ARG for a name the configuration does not have. */

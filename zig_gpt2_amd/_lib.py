@@ -51,7 +51,8 @@ class LmLayer(C.Structure):
                 ("lru_blocks", C.c_int), ("lru_conv", C.c_int), ("conv", C.c_int), ("decay_rank", C.c_int), ("gate_rank", C.c_int),
                 ("ff_act", C.c_int), ("router", C.c_int), ("keep_first", C.c_int), ("left_scale", C.c_float), ("right_scale", C.c_float),
                 ("lin_heads", C.c_int), ("lin_dim", C.c_int), ("lin_vdim", C.c_int), ("ff_limit", C.c_float), ("shared_width", C.c_int),
-                ("shared_limit", C.c_float)]
+                ("shared_limit", C.c_float), ("tau", C.c_float), ("softcap", C.c_float), ("qtemp_coef", C.c_float), ("qtemp_every", C.c_int),
+                ("dist_bias", C.c_int), ("route_groups", C.c_int), ("route_keep", C.c_int), ("route_scale", C.c_float), ("weights_of", C.c_int)]
 
 
 class LmConfig(C.Structure):
@@ -60,7 +61,7 @@ class LmConfig(C.Structure):
     _fields_ = [("vocab", sz), ("width", sz), ("n_layers", sz), ("layers", C.POINTER(LmLayer)), ("loop_start", C.c_int), ("loop_stop", C.c_int),
                 ("loop_times", C.c_int), ("norm_eps", C.c_float), ("max_tokens", sz), ("max_seqs", sz), ("max_step_tokens", sz),
                 ("page_tokens", sz), ("flags", C.c_uint), ("embed_scale", C.c_float), ("canon_taps", C.c_int), ("logit_scale", C.c_float),
-                ("logit_softcap", C.c_float)]
+                ("logit_softcap", C.c_float), ("residual_mult", C.c_float)]
 
 
 class LmEntry(C.Structure):
@@ -70,11 +71,14 @@ class LmEntry(C.Structure):
 
 
 LM_MIX_HGRN2, LM_MIX_LATENT_ATTENTION, LM_MIX_PARALLEL, LM_MIX_CHANNEL_DELTA, LM_MIX_WINDOW_LINEAR = 1, 2, 3, 4, 5
+LM_MIX_GLA, LM_MIX_ATTENTION = 6, 7
 LM_FF_NONE, LM_FF_DENSE, LM_FF_MOE = 0, 1, 2
 LM_ACT_GLU_SILU, LM_ACT_GELU, LM_ACT_GLU_CLIPPED = 0, 1, 2
 LM_ROUTE_SOFTMAX_ALL, LM_ROUTE_TOP_LOGITS, LM_ROUTE_SIGMOID_INPUT = 0, 1, 2
+LM_ROUTE_SIGMOID_GROUPS = 3
 LM_ROT_PLAIN, LM_ROT_YARN, LM_ROT_BANDS = 0, 1, 2
 LM_F32, LM_NO_GRAPH, LM_TIED_HEAD, LM_LOOP_READD, LM_SIDE_BY_SIDE, LM_SINUSOID_POSITIONS = 1, 2, 4, 8, 16, 32
+LM_TANH_NORMS, LM_EMBED_NORM = 64, 128
 
 # the layered-model tier (present in both libraries)
 LM_SIGNATURES = {

@@ -23,6 +23,12 @@
 // [heads][dim][vdim] state of the linear attention in the same block of sequence state; its keys (normed) and values go to the
 // paged cache as the other windowed attention's do.
 //
+// Designs whose norms are tanh(alpha v) * w + b keep a norm's three tensors together ([w | b | alpha]); such a norm needs no
+// statistic, so the norm behind a sublayer, the residual sum (times the design's factor) and the norm in front of the next
+// sublayer are one elementwise launch.  A layer that names another layer's weights is one more pass over that layer's tensors
+// with separate cache and state.  Their gated linear attention keeps its [heads][dim][vdim] state in the block of sequence
+// state; their attention caches the normed key heads and, as values, the projected ones.
+//
 // Latent attention runs in its absorbed form in prompts and in decoding alike: score_j = (W_uk^T q_nope) . c_j + q_rot . k_rot_j,
 // out = W_uv (sum_j p_j c_j) — only the latent c_j and the rotated key part are cached, and a portion of a prompt needs nothing
 // of the tokens before it but their cache rows.
@@ -82,6 +88,8 @@ struct LayerW {
     // in one vector, the whole-projection norms, the shared expert ([gate | up | gate logit] rows)
     bf16_t *ocat = nullptr, *sgu = nullptr, *sdown = nullptr;
     float *qkv_bias = nullptr, *qnorm = nullptr, *knorm = nullptr, *rnorm = nullptr, *obias = nullptr, *decay = nullptr;
+    // gated linear attention: the bias of the decay's second step;  attention: the heads' slopes of the distance bias
+    float *a2b = nullptr, *slopes = nullptr;
 };
 
 struct Pass {
@@ -188,6 +196,9 @@ struct zg_lm {
     int keep_pages = 0;   // pages that hold those first tokens: never returned while the sequence is open
     float embed_scale = 1.0f;
     bool side = false;          // ZG_LM_SIDE_BY_SIDE
+    bool tanh_norms = false;    // ZG_LM_TANH_NORMS: every norm pointer is a block [w | b | alpha]
+    float res_mult = 1.0f;      // ... and a sublayer's normed output enters the residual sum times this
+    float* embed_norm = nullptr;  // ZG_LM_EMBED_NORM
     float* pos_freq = nullptr;  // ZG_LM_SINUSOID_POSITIONS: frequency of every pair of channels
     int* page_table = nullptr;  // [NS][max_pages]
     std::vector<Slot> slots;
@@ -212,6 +223,7 @@ struct zg_lm {
     size_t trace_floats = 0;
     float last_step_ms = 0.0f, last_decode_ms = 0.0f;
     bool use_graph = true;
+    int step_keys = 0;  // positions the longest sequence of the running portion has reached (what its rows can see at most)
     hipGraphExec_t decode_graph[kGemvMaxRows + 1] = {};  // by rows of the step (one per entry)
 };
 
@@ -264,16 +276,26 @@ void layout(zg_lm* g, Bump& b) {
         t.init = init;
         T[name] = t;
     };
+    // a norm tanh(alpha v) * w + b: its three tensors side by side
+    auto norm3 = [&](const std::string& name, float*& p) {
+        p = b.take<float>(2 * W + 1);
+        vec_at(name, p, 0, W, INIT_PLAIN);
+        vec_at(name + ".b", p, W, W, INIT_OFFSET);
+        vec_at(name + ".alpha", p, 2 * W, 1, INIT_PLAIN);
+    };
+    const bool tn = g->tanh_norms;
     const size_t taps = g->canon;
     g->embed = b.take<bf16_t>(V * W);
     mat("embed", g->embed, 0, V, W);
+    if (tn && (g->cfg.flags & ZG_LM_EMBED_NORM)) norm3("embed.norm", g->embed_norm);
     if (g->cfg.flags & ZG_LM_TIED_HEAD) {
         g->head = g->embed;
     } else {
         g->head = b.take<bf16_t>(V * W);
         mat("head", g->head, 0, V, W);
     }
-    vec("final.norm", g->final_norm, W, g->side ? INIT_PLAIN : INIT_OFFSET);
+    if (tn) norm3("final.norm", g->final_norm);
+    else vec("final.norm", g->final_norm, W, g->side ? INIT_PLAIN : INIT_OFFSET);
     if (g->cfg.flags & ZG_LM_SINUSOID_POSITIONS) g->pos_freq = b.take<float>((W + 1) / 2);
     size_t max_t = 1, max_win = 0, max_win_few = 0;
     size_t max_proj = 1, max_qr = 1, max_q = 1, max_qa = 1, max_ctx = 1, max_o = 1, max_ff = 1, max_assign = 1, max_gu = 1, max_hb = 1, max_e = 1, max_att_part = 0, max_scan = 0;
@@ -281,8 +303,12 @@ void layout(zg_lm* g, Bump& b) {
         LayerW& L = g->layers[i];
         const zg_lm_layer& d = L.d;
         const std::string p = "l" + std::to_string(i) + ".";
-        vec(p + "norm1", L.norm1, W, g->side ? INIT_PLAIN : INIT_OFFSET);
-        if (g->side) {
+        if (d.weights_of > 0) continue;  // another layer's tensors
+        if (tn) {
+            norm3(p + "norm1", L.norm1);
+            norm3(p + "norm1b", L.norm1b);
+        } else vec(p + "norm1", L.norm1, W, g->side ? INIT_PLAIN : INIT_OFFSET);
+        if (g->side || tn) {
         } else {
             vec(p + "norm1b", L.norm1b, W, INIT_OFFSET);
             if (taps == 0) vec(p + "shift", L.shift, W, INIT_UNIT);
@@ -392,6 +418,40 @@ void layout(zg_lm* g, Bump& b) {
             mat(p + "mix.o", L.o, 0, W, HV);
             max_proj = std::max(max_proj, NP);
             max_t = std::max(max_t, std::max(CC, std::max(H * D, HV)));
+        } else if (d.mixer == ZG_LM_MIX_GLA) {
+            const size_t HD = H * D, HV = H * Vd, RA = d.decay_rank, NP = 2 * HD + 2 * HV + RA;
+            L.n_cat = (int)NP;
+            L.wcat = b.take<bf16_t>(NP * W);  // q | k | v | gate | the decay's first step
+            mat(p + "mix.q", L.wcat, 0, HD, W);
+            mat(p + "mix.k", L.wcat, HD, HD, W);
+            mat(p + "mix.v", L.wcat, 2 * HD, HV, W);
+            mat(p + "mix.g", L.wcat, 2 * HD + HV, HV, W);
+            mat(p + "mix.a1", L.wcat, 2 * HD + 2 * HV, RA, W);
+            L.a2 = b.take<bf16_t>(HD * RA);
+            mat(p + "mix.a2", L.a2, 0, HD, RA);
+            vec(p + "mix.a2.b", L.a2b, HD, INIT_OFFSET);
+            vec(p + "mix.norm", L.hnorm, Vd, INIT_PLAIN);
+            L.o = b.take<bf16_t>(W * HV);
+            mat(p + "mix.o", L.o, 0, W, HV);
+            max_proj = std::max(max_proj, NP);
+            max_t = std::max(max_t, HD);
+            max_scan = std::max(max_scan, HD * Vd + HD);
+            max_o = std::max(max_o, HV);
+        } else if (d.mixer == ZG_LM_MIX_ATTENTION) {
+            const size_t G = d.kv_heads, HD = H * D, GD = G * D, NP = HD + GD;
+            L.n_cat = (int)NP;
+            L.wcat = b.take<bf16_t>(NP * W);  // q | k (values reuse the key projection)
+            mat(p + "mix.q", L.wcat, 0, HD, W);
+            mat(p + "mix.k", L.wcat, HD, GD, W);
+            L.o = b.take<bf16_t>(W * HD);
+            mat(p + "mix.o", L.o, 0, W, HD);
+            L.slopes = b.take<float>(H);
+            max_proj = std::max(max_proj, NP);
+            max_o = std::max(max_o, HD);
+            // (a portion's score rows are as long as its longest sequence: what exceeds the bound below takes the general kernel)
+            const int cap = g->max_pages * g->P;
+            max_win = std::max(max_win, std::min(window_split_workspace((int)MS, (int)H, (int)D, cap, nullptr), (size_t)1 << 29));
+            max_win_few = std::max(max_win_few, window_split_workspace(kGemvMaxRows, (int)H, (int)D, cap, nullptr));
         } else if (d.mixer == ZG_LM_MIX_HGRN2) {
             const size_t HD = H * D, HV = H * Vd;
             L.qfv = b.take<bf16_t>((2 * HD + HV) * W);
@@ -430,7 +490,10 @@ void layout(zg_lm* g, Bump& b) {
             max_att_part = std::max(max_att_part, H * (KR + 2));
             max_o = std::max(max_o, HV);
         }
-        if (d.ff != ZG_LM_FF_NONE) {
+        if (d.ff != ZG_LM_FF_NONE && tn) {
+            norm3(p + "norm2", L.norm2);
+            norm3(p + "norm2b", L.norm2b);
+        } else if (d.ff != ZG_LM_FF_NONE) {
             vec(p + "norm2", L.norm2, W, g->side ? INIT_PLAIN : INIT_OFFSET);
             if (!g->side) vec(p + "norm2b", L.norm2b, W, INIT_OFFSET);
             if (taps && !g->side) vec(p + "canon2", L.canon2, W * taps, INIT_OFFSET);
@@ -456,12 +519,12 @@ void layout(zg_lm* g, Bump& b) {
             mat(p + "mlp.router", L.router, 0, E, W);
             if (d.router != ZG_LM_ROUTE_SIGMOID_INPUT)
                 vec(p + (d.router == ZG_LM_ROUTE_TOP_LOGITS ? "mlp.router.b" : "mlp.correction"), L.correction, E, INIT_OFFSET);
-            if (d.shared_width > 0) {  // the shared expert: gate | up rows and, behind them, the row of its gate logit
+            if (d.shared_width > 0) {  // the shared expert: gate | up rows and, behind them, the row of its gate logit (clipped form)
                 const size_t S = d.shared_width;
                 L.sgu = b.take<bf16_t>((2 * S + 1) * W);
                 mat(p + "mlp.shared.gate", L.sgu, 0, S, W);
                 mat(p + "mlp.shared.up", L.sgu, S, S, W);
-                mat(p + "mlp.shared.sg", L.sgu, 2 * S, 1, W);
+                if (d.ff_act == ZG_LM_ACT_GLU_CLIPPED) mat(p + "mlp.shared.sg", L.sgu, 2 * S, 1, W);
                 L.sdown = b.take<bf16_t>(W * S);
                 mat(p + "mlp.shared.down", L.sdown, 0, W, S);
                 max_t = std::max(max_t, std::max(2 * S + 1, W));
@@ -510,6 +573,9 @@ void layout(zg_lm* g, Bump& b) {
             sq += (size_t)(std::max(1, d.conv) - 1) * ((size_t)d.heads * d.dim + (size_t)d.kv_heads * (d.dim + d.vdim));
             ps.rec_off = sq;
             sq += (size_t)d.lin_heads * d.lin_dim * d.lin_vdim;
+        } else if (d.mixer == ZG_LM_MIX_GLA) {
+            ps.rec_off = sq;
+            sq += (size_t)d.heads * d.dim * d.vdim;
         }
     }
     g->seq_floats = sq;
@@ -520,6 +586,7 @@ void layout(zg_lm* g, Bump& b) {
         if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION) ps.cache = b.take<float>((size_t)g->n_pages * g->P * (d.kv_rank + d.rot_dim));
         if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_WINDOW_LINEAR)
             ps.cache = b.take<float>((size_t)g->n_pages * g->P * d.kv_heads * (d.dim + d.vdim));
+        if (d.mixer == ZG_LM_MIX_ATTENTION) ps.cache = b.take<float>((size_t)g->n_pages * g->P * d.kv_heads * 2 * d.dim);
     }
     // scratch
     g->x = b.take<float>(MS * W);
@@ -610,9 +677,9 @@ void rotary_table(const zg_lm_layer& d, std::vector<float>& freq, float& amp) {
 }
 
 int check_layer(const zg_lm_layer& d, size_t i, unsigned flags) {
-    ZG_REQUIRE(d.mixer >= ZG_LM_MIX_HGRN2 && d.mixer <= ZG_LM_MIX_WINDOW_LINEAR, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
+    ZG_REQUIRE(d.mixer >= ZG_LM_MIX_HGRN2 && d.mixer <= ZG_LM_MIX_ATTENTION, ZG_ERR_ARG, "layer %zu: unknown mixer %d", i, d.mixer);
     ZG_REQUIRE(d.heads >= 1 && d.dim >= 1 && d.vdim >= 1, ZG_ERR_ARG, "layer %zu: heads %d dim %d vdim %d", i, d.heads, d.dim, d.vdim);
-    if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_CHANNEL_DELTA || d.mixer == ZG_LM_MIX_WINDOW_LINEAR)
+    if (d.mixer == ZG_LM_MIX_PARALLEL || d.mixer == ZG_LM_MIX_CHANNEL_DELTA || d.mixer == ZG_LM_MIX_WINDOW_LINEAR || d.mixer == ZG_LM_MIX_ATTENTION)
         ZG_REQUIRE(d.kv_heads >= 1 && d.heads % d.kv_heads == 0, ZG_ERR_ARG, "layer %zu: %d heads on %d key heads", i, d.heads, d.kv_heads);
     if (d.mixer == ZG_LM_MIX_PARALLEL) {
         ZG_REQUIRE(d.vdim % 2 == 0, ZG_ERR_ARG, "layer %zu: %d value channels per head cannot be rotated in pairs", i, d.vdim);
@@ -638,6 +705,14 @@ int check_layer(const zg_lm_layer& d, size_t i, unsigned flags) {
                    d.vdim);
     } else if (d.mixer == ZG_LM_MIX_HGRN2) {
         ZG_REQUIRE(d.dim <= 256, ZG_ERR_UNSUPPORTED, "layer %zu: %d key channels per head of the recurrence (at most 256)", i, d.dim);
+    } else if (d.mixer == ZG_LM_MIX_GLA) {
+        ZG_REQUIRE(d.dim <= 256, ZG_ERR_UNSUPPORTED, "layer %zu: %d key channels per head of the recurrence (at most 256)", i, d.dim);
+        ZG_REQUIRE(d.tau > 0.0f && d.decay_rank >= 1, ZG_ERR_ARG, "layer %zu: decay root %g, inner size %d of its projection", i, d.tau, d.decay_rank);
+    } else if (d.mixer == ZG_LM_MIX_ATTENTION) {
+        ZG_REQUIRE(d.vdim == d.dim, ZG_ERR_ARG, "layer %zu: values reuse the key projection, so %d value channels cannot differ from %d key channels", i, d.vdim,
+                   d.dim);
+        ZG_REQUIRE(d.softcap >= 0.0f && d.qtemp_every >= 0 && d.window == 0, ZG_ERR_ARG, "layer %zu: score cap %g, query factor every %d, window %d", i,
+                   d.softcap, d.qtemp_every, d.window);
     } else {
         ZG_REQUIRE(d.rot_dim >= 0 && d.kv_rank >= 1 && d.q_rank >= 1, ZG_ERR_ARG, "layer %zu: rot_dim %d kv_rank %d q_rank %d", i, d.rot_dim,
                    d.kv_rank, d.q_rank);
@@ -654,16 +729,25 @@ int check_layer(const zg_lm_layer& d, size_t i, unsigned flags) {
     ZG_REQUIRE(d.ff != ZG_LM_FF_MOE || (d.experts >= 1 && d.experts <= 256 && d.top >= 1 && d.top <= d.experts), ZG_ERR_UNSUPPORTED,
                "layer %zu: %d experts, %d chosen (at most 256 experts)", i, d.experts, d.top);
     ZG_REQUIRE(d.ff_act >= ZG_LM_ACT_GLU_SILU && d.ff_act <= ZG_LM_ACT_GLU_CLIPPED && d.router >= ZG_LM_ROUTE_SOFTMAX_ALL &&
-                   d.router <= ZG_LM_ROUTE_SIGMOID_INPUT,
+                   d.router <= ZG_LM_ROUTE_SIGMOID_GROUPS,
                ZG_ERR_ARG, "layer %zu: expert activation %d, router rule %d", i, d.ff_act, d.router);
     if (d.ff == ZG_LM_FF_MOE && !(flags & ZG_LM_SIDE_BY_SIDE))
-        ZG_REQUIRE(d.ff_act != ZG_LM_ACT_GLU_CLIPPED && d.router != ZG_LM_ROUTE_SIGMOID_INPUT && d.shared_width == 0, ZG_ERR_UNSUPPORTED,
-                   "layer %zu: the clipped activation, the input-weighted router and the shared expert are built for side-by-side sublayers", i);
+        ZG_REQUIRE(d.ff_act != ZG_LM_ACT_GLU_CLIPPED && d.router != ZG_LM_ROUTE_SIGMOID_INPUT && (d.shared_width == 0 || (flags & ZG_LM_TANH_NORMS)),
+                   ZG_ERR_UNSUPPORTED,
+                   "layer %zu: the clipped activation and the input-weighted router are built for side-by-side sublayers, a shared expert for those or "
+                   "for the norms without statistics",
+                   i);
+    if (d.ff == ZG_LM_FF_MOE && d.router == ZG_LM_ROUTE_SIGMOID_GROUPS) {
+        const int ng = std::max(1, d.route_groups), nk = d.route_keep >= 1 ? d.route_keep : ng;
+        ZG_REQUIRE(d.experts % ng == 0 && nk <= ng && d.top <= nk * (d.experts / ng) && d.route_scale >= 0.0f, ZG_ERR_ARG,
+                   "layer %zu: %d experts in %d groups, %d groups kept, %d chosen, weight factor %g", i, d.experts, ng, nk, d.top, d.route_scale);
+    }
     if (d.ff == ZG_LM_FF_MOE && d.ff_act == ZG_LM_ACT_GLU_CLIPPED)
         ZG_REQUIRE(d.ff_limit > 0.0f && (d.shared_width == 0 || d.shared_limit > 0.0f), ZG_ERR_ARG, "layer %zu: clip %g (shared expert: %g)", i, d.ff_limit,
                    d.shared_limit);
-    ZG_REQUIRE(d.shared_width >= 0 && (d.shared_width == 0 || d.ff_act == ZG_LM_ACT_GLU_CLIPPED), ZG_ERR_UNSUPPORTED,
-               "layer %zu: a shared expert needs the clipped gated activation", i);
+    ZG_REQUIRE(d.shared_width >= 0 && (d.shared_width == 0 || d.ff_act == ZG_LM_ACT_GLU_CLIPPED ||
+                                       (d.ff_act == ZG_LM_ACT_GLU_SILU && (flags & ZG_LM_TANH_NORMS))),
+               ZG_ERR_UNSUPPORTED, "layer %zu: a shared expert needs a gated activation", i);
     return ZG_OK;
 }
 
@@ -683,6 +767,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
     const bool readd = (g->cfg.flags & ZG_LM_LOOP_READD) && g->cfg.loop_times > 1;
     ZG_TRY(launch_embed(g->embed, d_ids, g->x, readd ? g->x0 : nullptr, g->embed_scale, M, W, g->V, g->flag, d_pos, g->pos_freq, s));
     const bool side = g->side;
+    const bool tnorm = g->tanh_norms;
     // side-by-side sublayers: the sums a layer leaves for the next layer's norm kernel to add
     OpenSums pend;
     auto copy_trace = [&](int p) -> int {
@@ -700,6 +785,10 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         return launch_causal_conv(c, M, n_ent, single, d_off, d_slot, d_estart, d_elen, d_eslot, s);
     };
     bool h_ready = false;  // g->h already holds this pass's shifted norm (written by the previous pass's fused tail)
+    if (tnorm) {  // the norm behind the embedding (in place) and the first pass's norm; every later one rides behind a sublayer's sum
+        ZG_TRY(launch_tanh_norm(g->x, g->embed_norm, g->layers[g->passes[0].layer].norm1, nullptr, g->h, M, W, s));
+        h_ready = true;
+    }
     for (int p = 0; p < g->n_passes; ++p) {
         const Pass& ps = g->passes[p];
         const LayerW& L = g->layers[ps.layer];
@@ -831,6 +920,47 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             lin = Linear();
             lin.A = g->td; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));
+        } else if (d.mixer == ZG_LM_MIX_GLA) {
+            const int HD = H * D, HV = H * Vd, RA = d.decay_rank, NP = L.n_cat;
+            const int og = 2 * HD + HV, oa = og + HV;  // columns of the output gate and of the decay's first step
+            lin = Linear();
+            lin.A = hin; lin.lda = W; lin.B = L.wcat; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            lin = Linear();  // the decay's second step
+            lin.A = g->proj + oa; lin.lda = NP; lin.B = L.a2; lin.ldb = RA; lin.C = g->tb; lin.ldc = HD; lin.M = M; lin.N = HD; lin.K = RA;
+            ZG_TRY(launch_linear(lin, f32, s));
+            GlaGate gate;
+            gate.z = g->tb; gate.ldz = HD; gate.z_bias = L.a2b; gate.inv_tau = 1.0f / d.tau; gate.q_scale = 1.0f / sqrtf((float)D);
+            ZG_TRY(launch_hgrn2_scan(g->proj, NP, g->o, HV, g->seq_state + ps.rec_off, g->seq_floats, d_estart, d_elen, d_eslot, n_ent, M, H, D, Vd,
+                                     nullptr, nullptr, g->scan_ws, g->scan_ws_floats, s, nullptr, &gate));
+            ZG_TRY(launch_norm_gate(g->o, HV, H, Vd, M, L.hnorm, eps, g->proj + og, NP, s, 1.0f, true));
+            lin = Linear();
+            lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
+            ZG_TRY(launch_linear(lin, f32, s));
+        } else if (d.mixer == ZG_LM_MIX_ATTENTION) {
+            const int G = d.kv_heads, HD = H * D, NP = L.n_cat;
+            ScoreShape shape;
+            shape.cap = d.softcap;
+            shape.slope = d.dist_bias ? L.slopes : nullptr;
+            lin = Linear();
+            lin.A = hin; lin.lda = W; lin.B = L.wcat; lin.ldb = W; lin.C = g->proj; lin.ldc = NP; lin.M = M; lin.N = NP; lin.K = W;
+            ZG_TRY(launch_linear(lin, f32, s));
+            ZG_TRY(launch_head_norm_prep(g->proj, NP, M, H, G, D, eps, d.qtemp_coef, d.qtemp_every, d_pos, d_slot, g->page_table, g->max_pages, g->P,
+                                         ps.cache, s));
+            // rows of the score workspace: as long as the longest sequence of this portion (a captured decode step replays at any
+            // length, so it takes the cache's capacity)
+            const int all_keys = g->max_pages * g->P;
+            const int key_cap = (single || capturing) ? all_keys : std::min(all_keys, (g->step_keys + 63) / 64 * 64);
+            bool split = false;
+            ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HD, M, H, G, D, D, d.scale, 0, 0, nullptr, nullptr, nullptr, d_pos, d_slot,
+                                                 g->page_table, g->max_pages, g->P, ps.cache, key_cap, g->win_ws, g->win_ws_floats, d_estart, d_elen,
+                                                 n_ent, s, &split, nullptr, 0, 1.0f, shape));
+            if (!split)
+                ZG_TRY(launch_window_attention(g->proj, NP, g->o, HD, M, H, G, D, D, d.scale, 0, 0, nullptr, nullptr, nullptr, d_pos, d_slot,
+                                               g->page_table, g->max_pages, g->P, ps.cache, s, shape));
+            lin = Linear();
+            lin.A = g->o; lin.lda = HD; lin.B = L.o; lin.ldb = HD; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HD;
+            ZG_TRY(launch_linear(lin, f32, s));
         } else if (d.mixer == ZG_LM_MIX_HGRN2) {
             const int HD = H * D, HV = H * Vd, NP = 2 * HD + HV;
             lin = Linear();
@@ -873,6 +1003,96 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             lin.A = g->o; lin.lda = HV; lin.B = L.o; lin.ldb = HV; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = HV;
             ZG_TRY(launch_linear(lin, f32, s));
         }
+        if (tnorm) {  // norms without statistics: every sum behind a sublayer carries the next sublayer's norm
+            const float* next_norm = p + 1 < g->n_passes ? g->layers[g->passes[p + 1].layer].norm1 : nullptr;
+            SumParts part;
+            part.a = g->y;
+            // steps of few rows: the router's workgroups do the sum and the norms in front of them themselves
+            RoutePre pre;
+            const bool pre_routed = few && d.ff == ZG_LM_FF_MOE && W <= kRouteFuseWidth;
+            if (pre_routed) {
+                pre.x = g->x; pre.y = part; pre.nb = L.norm1b; pre.mult = g->res_mult; pre.nn = L.norm2; pre.h = g->h;
+            } else {
+                ZG_TRY(launch_tanh_sum_norm(g->x, part, L.norm1b, g->res_mult, d.ff != ZG_LM_FF_NONE ? L.norm2 : next_norm, g->h, M, W, s));
+            }
+            const int F = d.ff_width;
+            part = SumParts();
+            if (d.ff == ZG_LM_FF_DENSE) {
+                lin = Linear();
+                lin.A = g->h; lin.lda = W; lin.B = L.up; lin.ldb = W; lin.C = g->u; lin.ldc = F; lin.M = M; lin.N = F; lin.K = W; lin.act = ACT_RELU2;
+                ZG_TRY(launch_linear(lin, f32, s));
+                lin = Linear();
+                lin.A = g->u; lin.lda = F; lin.B = L.down; lin.ldb = F; lin.C = g->y; lin.ldc = W; lin.M = M; lin.N = W; lin.K = F;
+                ZG_TRY(launch_linear(lin, f32, s));
+                part.a = g->y;
+            } else if (d.ff == ZG_LM_FF_MOE) {
+                const int E = d.experts, top = d.top, NA = M * top;
+                const bool glu = d.ff_act == ZG_LM_ACT_GLU_SILU;
+                const int UF = glu ? 2 * F : F;
+                ZG_TRY(launch_route(g->h, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s, d.route_groups, d.route_keep,
+                                    d.route_scale != 0.0f ? d.route_scale : 1.0f, pre_routed ? &pre : nullptr));
+                Linear up, dn;
+                up.A = g->h; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
+                up.N = UF; up.K = W;
+                if (!glu) up.act = ACT_GELU_ERF;
+                dn.A = g->hb; dn.lda = F; dn.B = L.edown; dn.ldb = F; dn.b_zoff = (long long)W * F; dn.C = g->ye; dn.ldc = W; dn.N = W; dn.K = F;
+                if (few) {  // one batch per assignment, its expert's matrices looked up on the device
+                    up.M = dn.M = 1; up.nz = dn.nz = NA; up.z_group = dn.z_group = g->pick;
+                    up.c_zoff = UF; dn.c_zoff = W;
+                } else {  // assignments sorted by expert, grouped products
+                    ZG_TRY(launch_group(g->pick, NA, E, g->grp_off, g->sorted, g->inv, s));
+                    up.M = dn.M = NA; up.a_rows = g->sorted; up.grp_off = dn.grp_off = g->grp_off; up.n_groups = dn.n_groups = E;
+                }
+                part.exp = g->ye; part.exp_w = g->wt; part.inv = few ? nullptr : g->inv; part.top = top;
+                if (few && glu && d.shared_width > 0) {
+                    // steps of few rows: the expert every token uses rides in the launches of the chosen experts, a batch per row; the
+                    // gated activation is applied where the second products read their rows
+                    const int S = d.shared_width;
+                    Linear sup, sdn;
+                    sup.A = g->h; sup.lda = W; sup.a_zoff = W; sup.B = L.sgu; sup.ldb = W; sup.C = g->tb; sup.ldc = 2 * S; sup.c_zoff = 2 * S;
+                    sup.M = 1; sup.nz = M; sup.N = 2 * S; sup.K = W;
+                    ZG_TRY(launch_linear_pair(up, sup, f32, s));
+                    dn.A = g->gu_buf; dn.lda = 2 * F; dn.a_glu = F;
+                    sdn.A = g->tb; sdn.lda = 2 * S; sdn.a_zoff = 2 * S; sdn.a_glu = S; sdn.B = L.sdown; sdn.ldb = S; sdn.C = g->td; sdn.ldc = W;
+                    sdn.c_zoff = W; sdn.M = 1; sdn.nz = M; sdn.N = W; sdn.K = S;
+                    ZG_TRY(launch_linear_pair(dn, sdn, f32, s));
+                    part.b = g->td;
+                    ZG_TRY(launch_tanh_sum_norm(g->x, part, L.norm2b, g->res_mult, next_norm, g->h, M, W, s));
+                    h_ready = next_norm != nullptr;
+                    ZG_TRY(copy_trace(p));
+                    continue;
+                }
+                ZG_TRY(launch_linear(up, f32, s));
+                if (!glu) {  // the first product's epilogue has applied the activation
+                    dn.A = g->gu_buf; dn.lda = F;
+                } else if (few) {  // the gated activation is applied where the second product reads its rows
+                    dn.A = g->gu_buf; dn.lda = 2 * F; dn.a_glu = F;
+                } else {
+                    ZG_TRY(launch_glu(g->gu_buf, g->hb, NA, F, s));
+                }
+                ZG_TRY(launch_linear(dn, f32, s));
+                if (d.shared_width > 0) {  // the expert every token uses
+                    const int S = d.shared_width;
+                    lin = Linear();
+                    lin.A = g->h; lin.lda = W; lin.B = L.sgu; lin.ldb = W; lin.C = g->tb; lin.ldc = 2 * S; lin.M = M; lin.N = 2 * S; lin.K = W;
+                    ZG_TRY(launch_linear(lin, f32, s));
+                    lin = Linear();
+                    lin.B = L.sdown; lin.ldb = S; lin.C = g->td; lin.ldc = W; lin.M = M; lin.N = W; lin.K = S;
+                    if (M <= 2) {  // the activation where the second product reads its rows (more rows: every workgroup would redo it)
+                        lin.A = g->tb; lin.lda = 2 * S; lin.a_glu = S;
+                    } else {
+                        ZG_TRY(launch_glu(g->tb, g->tc, M, S, s));
+                        lin.A = g->tc; lin.lda = S;
+                    }
+                    ZG_TRY(launch_linear(lin, f32, s));
+                    part.b = g->td;
+                }
+            }
+            if (d.ff != ZG_LM_FF_NONE) ZG_TRY(launch_tanh_sum_norm(g->x, part, L.norm2b, g->res_mult, next_norm, g->h, M, W, s));
+            h_ready = next_norm != nullptr;
+            ZG_TRY(copy_trace(p));
+            continue;
+        }
         if (side) {  // the feed-forward beside the mixer, on the second norm of the same x
             const int F = d.ff_width;
             const float* fin = g->hc;
@@ -887,7 +1107,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
                 const int E = d.experts, top = d.top, NA = M * top;
                 const int UF = d.ff_act == ZG_LM_ACT_GELU ? F : 2 * F;
                 const bool on_input = d.router == ZG_LM_ROUTE_SIGMOID_INPUT;  // the router's score multiplies the expert's input
-                ZG_TRY(launch_route(fin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s));
+                ZG_TRY(launch_route(fin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s, d.route_groups, d.route_keep,
+                                    d.route_scale != 0.0f ? d.route_scale : 1.0f));
                 Linear up, dn;
                 up.A = fin; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
                 up.N = UF; up.K = W;
@@ -980,7 +1201,8 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             const int E = d.experts, top = d.top, NA = M * top;
             const bool glu = d.ff_act == ZG_LM_ACT_GLU_SILU;
             const int UF = glu ? 2 * F : F;
-            ZG_TRY(launch_route(hin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s));
+            ZG_TRY(launch_route(hin, M, W, L.router, L.correction, E, top, g->pick, g->wt, d.router, s, d.route_groups, d.route_keep,
+                                d.route_scale != 0.0f ? d.route_scale : 1.0f));
             Linear up, dn;
             up.A = hin; up.lda = W; up.a_div = top; up.B = L.gu; up.ldb = W; up.b_zoff = (long long)UF * W; up.C = g->gu_buf; up.ldc = UF;
             up.N = UF; up.K = W;
@@ -1008,7 +1230,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
         ZG_TRY(copy_trace(p));
     }
     // the rows the last tokens of the entries left for the token shift of their successors
-    if (!canon && !side) ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
+    if (!canon && !side && !tnorm) ZG_TRY(launch_commit_rows(g->shift_state, (size_t)g->n_passes * W, g->last_h, W, d_eslot, n_ent, W, g->n_passes, W, (size_t)NS * W, s));
 
     return ZG_OK;
 }
@@ -1026,8 +1248,10 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
     int* row_off = g->h_meta + meta_row_off(g);
     std::vector<std::pair<int, size_t>> wants;  // (row of the portion, output row)
     int r = 0;
+    g->step_keys = 0;
     for (int e = 0; e < n_ent; ++e) {
         const Piece& pc = pieces[e];
+        g->step_keys = std::max(g->step_keys, pc.pos0 + pc.n);
         ent_start[e] = r;
         ent_len[e] = pc.n;
         ent_slot[e] = pc.slot;
@@ -1081,7 +1305,8 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
             // so the twin is free again when the next batch fills it)
             for (int j = 0; j < nw; ++j) want_rows[j] = wants[w0 + j].first;
             ZG_HIP(hipMemcpyAsync(g->meta + 5 * (size_t)MS, want_rows, nw * sizeof(int), hipMemcpyHostToDevice, s));
-            ZG_TRY(launch_norm_gather(g->x, d_want, g->final_norm, eps, g->hn, nw, W, g->side, s));
+            if (g->tanh_norms) ZG_TRY(launch_tanh_norm(g->x, nullptr, g->final_norm, d_want, g->hn, nw, W, s));
+            else ZG_TRY(launch_norm_gather(g->x, d_want, g->final_norm, eps, g->hn, nw, W, g->side, s));
             Linear lin;
             lin.A = g->hn; lin.lda = W; lin.B = g->head; lin.ldb = W; lin.C = g->logits; lin.ldc = g->V; lin.M = nw; lin.N = g->V; lin.K = W;
             if ((g->cfg.logit_scale != 0.0f && g->cfg.logit_scale != 1.0f) || g->cfg.logit_softcap > 0.0f) {
@@ -1240,6 +1465,8 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     g->logit_rows = std::min(g->MS, 256);
     g->canon = config->canon_taps;
     g->side = (config->flags & ZG_LM_SIDE_BY_SIDE) != 0;
+    g->tanh_norms = (config->flags & ZG_LM_TANH_NORMS) != 0;
+    g->res_mult = config->residual_mult != 0.0f ? config->residual_mult : 1.0f;
     g->embed_scale = config->embed_scale != 0.0f ? config->embed_scale : 1.0f;
     int status = ZG_OK;
     for (size_t i = 0; i < config->n_layers && status == ZG_OK; ++i) {
@@ -1249,6 +1476,37 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
         g->layers.push_back(L);
     }
     g->cfg.layers = nullptr;
+    // a layer that runs another layer's tensors: follow the chain to the layer that owns them
+    std::vector<int> owner(config->n_layers);
+    for (size_t i = 0; i < config->n_layers && status == ZG_OK; ++i) {
+        size_t j = i, hops = 0;
+        while (g->layers[j].d.weights_of > 0 && status == ZG_OK) {
+            const int w = g->layers[j].d.weights_of - 1;
+            if (w < 0 || (size_t)w >= config->n_layers || (size_t)w == j || ++hops > config->n_layers) {
+                set_error("lm_create: layer %zu names the weights of layer %d", j, w);
+                status = ZG_ERR_ARG;
+                break;
+            }
+            j = (size_t)w;
+        }
+        owner[i] = (int)j;
+        if (status == ZG_OK && j != i) {
+            const zg_lm_layer &a = g->layers[i].d, &o = g->layers[j].d;
+            if (a.mixer != o.mixer || a.heads != o.heads || a.dim != o.dim || a.vdim != o.vdim || a.kv_heads != o.kv_heads || a.ff != o.ff ||
+                a.ff_width != o.ff_width || a.experts != o.experts || a.top != o.top || a.shared_width != o.shared_width) {
+                set_error("lm_create: layer %zu names the weights of layer %zu, whose sizes differ", i, j);
+                status = ZG_ERR_ARG;
+            }
+        }
+    }
+    if (status == ZG_OK && g->tanh_norms && (g->side || g->canon != 0 || (config->flags & ZG_LM_LOOP_READD))) {
+        set_error("lm_create: the norms without statistics stand in sequential sublayers, without input convolution or re-added embedding");
+        status = ZG_ERR_UNSUPPORTED;
+    }
+    if (status == ZG_OK && !g->tanh_norms && (config->flags & ZG_LM_EMBED_NORM)) {
+        set_error("lm_create: a norm behind the embedding is built for the norms without statistics");
+        status = ZG_ERR_UNSUPPORTED;
+    }
     if (status == ZG_OK && g->side && (g->canon != 0 || config->loop_times > 1)) {
         set_error("lm_create: side-by-side sublayers have no input convolution and no looped span");
         status = ZG_ERR_UNSUPPORTED;
@@ -1272,7 +1530,7 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     }
     auto add = [&](int layer) {
         Pass ps;
-        ps.layer = layer;
+        ps.layer = owner[layer];
         g->passes.push_back(ps);
     };
     for (int i = 0; i < a; ++i) add(i);
@@ -1287,7 +1545,8 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
     bool attends = false, bounded = true;
     for (const Pass& ps : g->passes) {
         const zg_lm_layer& d = g->layers[ps.layer].d;
-        if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION || (d.mixer == ZG_LM_MIX_PARALLEL && d.window == 0)) attends = true, bounded = false;
+        if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION || d.mixer == ZG_LM_MIX_ATTENTION || (d.mixer == ZG_LM_MIX_PARALLEL && d.window == 0))
+            attends = true, bounded = false;
         if (d.mixer == ZG_LM_MIX_PARALLEL && d.window > 0) {
             attends = true;
             g->keep_tokens = std::max(g->keep_tokens, d.window);
@@ -1350,12 +1609,18 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
         ZG_LM_TRY_HIP(hipMemcpy(g->pos_freq, pf.data(), pf.size() * sizeof(float), hipMemcpyHostToDevice));
     }
     for (LayerW& L : g->layers)
-        if (L.d.mixer == ZG_LM_MIX_WINDOW_LINEAR && L.d.conv == 0) {  // no convolution: one tap of weight one
+        if (L.d.mixer == ZG_LM_MIX_WINDOW_LINEAR && L.d.conv == 0 && L.d.weights_of == 0) {  // no convolution: one tap of weight one
             const size_t n = (size_t)L.d.heads * L.d.dim + (size_t)L.d.kv_heads * (L.d.dim + L.d.vdim);
             ones_kernel<<<(unsigned)((n + 255) / 256), 256, 0, g->stream>>>(L.convw, n);
         }
     for (LayerW& L : g->layers)
-        if (L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION || L.d.mixer == ZG_LM_MIX_PARALLEL) {
+        if (L.d.mixer == ZG_LM_MIX_ATTENTION && L.slopes) {  // head h loses 2^(-8 (h + 1) / heads) per position of distance
+            std::vector<float> sl(L.d.heads);
+            for (int h = 0; h < L.d.heads; ++h) sl[h] = (float)pow(2.0, -8.0 * (h + 1) / (double)L.d.heads);
+            ZG_LM_TRY_HIP(hipMemcpy(L.slopes, sl.data(), sl.size() * sizeof(float), hipMemcpyHostToDevice));
+        }
+    for (LayerW& L : g->layers)
+        if ((L.d.mixer == ZG_LM_MIX_LATENT_ATTENTION || L.d.mixer == ZG_LM_MIX_PARALLEL) && L.d.weights_of == 0) {
             std::vector<float> freq;
             rotary_table(L.d, freq, L.rot_amp);
             ZG_LM_TRY_HIP(hipMemcpy(L.rot_freq, freq.data(), std::max<size_t>(1, L.d.rot_dims / 2) * sizeof(float), hipMemcpyHostToDevice));

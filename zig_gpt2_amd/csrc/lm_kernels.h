@@ -51,6 +51,9 @@ struct Linear {
 // Picks the row-vector kernel (few rows: decode) or the tiled matrix-core kernel (prompt portions).
 int launch_linear(const Linear& L, bool f32, hipStream_t s);
 constexpr int kGemvMaxRows = 8;
+// Two products of one-row batches (M == 1 each) in ONE launch of the row-vector kernel; whatever does not fit that form runs as two
+// launches.  Neither product may read what the other writes.
+int launch_linear_pair(const Linear& a, const Linear& b, bool f32, hipStream_t s);
 
 // ------------------------------------------------------------------------------------------------ norms, embedding, shift
 // x[m] = table[ids[m]] (bf16 -> fp32); an id outside [0, vocab) raises *flag (pinned or device int) and yields a zero row.
@@ -99,6 +102,21 @@ int launch_add_two(float* x, const OpenSums& add, int M, int W, hipStream_t s);
 // In place over `rows` rows of `width` floats with row stride ld: v / rms(v) * w  (a plain weight; per-head norms)
 int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s);
 
+// Norms without statistics: n(v) = tanh(alpha v) * w + b.  A norm's tensors lie together, nw = [w (W) | b (W) | alpha (1)].
+// out[j] = n(x[rows ? rows[j] : j]);  pre != null (rows == null): x[j] <- pre(x[j]) first, in place (a norm behind the embedding).
+int launch_tanh_norm(float* x, const float* pre, const float* nw, const int* rows, float* out, int n_rows, int W, hipStream_t s);
+// What a sublayer left, summed in a fixed order:  a[m] + sum_k exp_w[m top + k] * exp[inv ? inv[m top + k] : m top + k] + b[m]
+// (any part may be null; the experts' rows in choice order).
+struct SumParts {
+    const float *a = nullptr, *exp = nullptr, *exp_w = nullptr;
+    const int* inv = nullptr;
+    int top = 0;
+    const float* b = nullptr;
+};
+// x[m] += mult * nb(sum of the parts);  h[m] = nn(x[m])   (nn / h may be null): the norm behind a sublayer, the residual sum and
+// the norm in front of the next sublayer in one launch.
+int launch_tanh_sum_norm(float* x, const SumParts& y, const float* nb, float mult, const float* nn, float* h, int M, int W, hipStream_t s);
+
 // ------------------------------------------------------------------------------------------------ gated linear recurrence (HGRN2)
 // proj rows are [q (H D) | f (H D) | v (H V)] as the fused projection left them; the gates are activated where the scan stages
 // them:  q <- silu(q);   f <- low + (1 - low) * sigmoid(f + bias)
@@ -107,9 +125,18 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
 // M: rows of the step.  ws (may be null): workspace for the chunk-parallel form of long steps, (M / 64 + n_entries) * (H D V + H D) floats.
 // decay != null: linear attention with one fixed decay per head on the same machinery — proj rows [q (H D) | k (H D) | v (H V)], all
 // three through silu on their way in:  S <- decay[h] S + k_t v_t^T, o_t = S^T q_t   (bias / low unused).
+// gla != null: gated linear attention with a decay per key channel on the same machinery — proj rows [q (H D) | k (H D) | v (H V)]
+// taken as they are, q times q_scale;  f = sigmoid(z + z_bias)^inv_tau, z rows [H D] with stride ldz (fp32 logarithm and
+// exponential);  S <- diag(f) S + k_t v_t^T, o_t = S^T q_t.
+struct GlaGate {
+    const float* z = nullptr;
+    int ldz = 0;
+    const float* z_bias = nullptr;
+    float inv_tau = 1.0f, q_scale = 1.0f;
+};
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
                       const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
-                      float* ws, size_t ws_floats, hipStream_t s, const float* decay = nullptr);
+                      float* ws, size_t ws_floats, hipStream_t s, const float* decay = nullptr, const GlaGate* gla = nullptr);
 
 // ------------------------------------------------------------------------------------------------ latent attention
 // Rotary table of one layer: freq[i] for the rot_dims / 2 pairs (YaRN blend applied on the host) and the amplitude factor.
@@ -179,9 +206,21 @@ int launch_window_prep(float* proj, int ld, int M, int H, int G, int D, int V, R
 // (window 0: all j <= pos).  sink / talk may be null (no sink / no mix).
 // keep_first > 0: beyond the window the first keep_first positions of the sequence stay visible (a row's keys are then numbered
 // kept tokens first, then the window).  vfreq == null: values are cached unrotated and nothing is turned back.
+// shape: what becomes of a scaled score before the softmax — capped (cap > 0: cap tanh(s / cap)), then less slope[h] per position
+// of distance between the query and the key (slope != null).
+struct ScoreShape {
+    float cap = 0.0f;
+    const float* slope = nullptr;  // [H]
+};
 int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                             int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
-                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s);
+                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s,
+                            ScoreShape shape = ScoreShape());
+// The prep of attention whose q and k are divided by their root mean square PER HEAD (no weight) and whose values are the
+// un-normalised key heads: rows qk [q (H D) | k (G D)]; q <- q / rms(q) * (1 + qt_coef ln(floor((pos + 1) / qt_every) + 1)) in place (qt_every 0:
+// no factor); the token's cache row [G D | G D] receives k / rms(k) and, behind it, k itself.
+int launch_head_norm_prep(float* qk, int ld, int M, int H, int G, int D, float eps, float qt_coef, int qt_every, const int* row_pos,
+                          const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s);
 // The prep of attention without rotation whose q and k are normed over the whole projection: rows qkv [q (H D) | k (G D) | v (G V)];
 // q <- q / rms(q) * wq in place (rms over all H D entries), k / rms(k) * wk and v into the token's cache row [G D | G V].
 // Steps of one row per entry: the convolution `a` over the channels q | k | v (its tails moved on) and the prep below in one launch,
@@ -204,7 +243,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
                                   int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
                                   size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken,
-                                  const float* out_gate = nullptr, int ld_gate = 0, float out_factor = 1.0f);
+                                  const float* out_gate = nullptr, int ld_gate = 0, float out_factor = 1.0f, ScoreShape shape = ScoreShape());
 // (out_gate != null: a taken step multiplies the result by sigmoid(out_gate[m][.]) * out_factor where the shares are added)
 
 // ------------------------------------------------------------------------------------------------ real-gated linear recurrent unit
@@ -228,15 +267,31 @@ int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const 
                       const int* ent_slot, int n_entries, hipStream_t s);
 // In place over M * rows_per_m vectors of `width` floats: v / rms(v) * w * sigmoid(gate) * factor (gate laid out like v, row stride
 // ldg).  w == null: no norm, the gate and the factor only.
+// gate_silu: the gate is silu(gate) instead of sigmoid(gate).
 int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s,
-                     float factor = 1.0f);
+                     float factor = 1.0f, bool gate_silu = false);
 
 // ------------------------------------------------------------------------------------------------ mixture of experts
 // Per row: z = router . g (fp32), s = softmax(z), the `top` experts by s + correction (lowest index wins a tie), weights s.
 // top_logits: z += correction (a bias), the `top` largest z (lowest index wins a tie), weights = softmax over the chosen z.
 // rule ZG_LM_ROUTE_SIGMOID_INPUT: the `top` largest z (= the largest sigmoid scores; lowest index wins a tie), weights sigmoid(z).
+// rule ZG_LM_ROUTE_SIGMOID_GROUPS: s = sigmoid(z), experts ranked by r = s + correction; the expert list is cut into `groups`
+// contiguous blocks of equal size, a block ranks by r of its best plus r of its second-best expert, experts outside the `keep`
+// top-ranked blocks get r = -inf; the `top` highest r win (lowest index wins a tie); weights s / (sum of the winners' s + 1e-20)
+// * out_scale.
+// pre != null (norms without statistics, widths up to kRouteFuseWidth): the routing workgroup of a row first does what
+// launch_tanh_sum_norm would — x[m] += mult * nb(sum of y's parts), h[m] = nn(x[m]) with h == g — and routes on the result.
+struct RoutePre {
+    float* x = nullptr;
+    SumParts y;
+    const float* nb = nullptr;
+    float mult = 1.0f;
+    const float* nn = nullptr;
+    float* h = nullptr;
+};
+constexpr int kRouteFuseWidth = 8192;
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 int rule, hipStream_t s);
+                 int rule, hipStream_t s, int groups = 1, int keep = 1, float out_scale = 1.0f, const RoutePre* pre = nullptr);
 // Sort the M * top assignments by expert: grp_off[E + 1], sorted[p] = assignment at sorted position p, inv[a] = position of a.
 int launch_group(const int* pick, int n_assign, int E, int* grp_off, int* sorted, int* inv, hipStream_t s);
 // h[p][j] = silu(gu[p][j]) * gu[p][F + j]

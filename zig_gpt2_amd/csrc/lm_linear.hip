@@ -11,6 +11,8 @@
 // an index array (the expert of an assignment), and row groups sorted by expert with their offsets in device memory.
 #include <stdlib.h>
 
+#include <algorithm>
+
 #include <type_traits>
 
 #include "lm_kernels.h"
@@ -91,8 +93,8 @@ __device__ __forceinline__ f32x4 load_a4(const float* a, int k, int K, bool vec)
 
 // ------------------------------------------------------------------------------------------------ few rows
 template <int MR>
-__global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
-    const int z = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__device__ __forceinline__ void gemv_body(const LinArgs& p, const int z) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 8 + wave * 2;
     if (n0 >= p.N) return;
     const bf16_t* B = p.B + (long long)(p.z_group ? p.z_group[z] : z) * p.b_zoff;
@@ -171,6 +173,18 @@ __global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
             if (two) C[(long long)m * p.ldc + n0 + 1] = apply_act(s1, p);
         }
     }
+}
+
+template <int MR>
+__global__ __launch_bounds__(256) void lm_gemv_kernel(const LinArgs p) {
+    gemv_body<MR>(p, blockIdx.z);
+}
+
+// Two products of one-row batches in one launch: batches [0, nz_a) are product a's, the rest product b's (the chosen experts and the
+// expert every token uses read the same rows; a decode step saves a dependent launch per product).
+__global__ __launch_bounds__(256) void lm_gemv_pair_kernel(const LinArgs a, const LinArgs b, int nz_a) {
+    if ((int)blockIdx.z < nz_a) gemv_body<1>(a, blockIdx.z);
+    else gemv_body<1>(b, blockIdx.z - nz_a);
 }
 
 // The same for long rows (K >= 1536; at 1024 columns half the lanes of a quarter idle and it measured 6 % slower): a workgroup owns two weight rows and its four waves split K into quarters, so a matrix of
@@ -441,10 +455,28 @@ __global__ __launch_bounds__(256) void lm_gemm_kernel(const LinArgs p) {
 
 }  // namespace
 
-int launch_linear(const Linear& L, bool f32, hipStream_t s) {
-    if (L.M <= 0 || L.N <= 0 || L.nz <= 0) return ZG_OK;
-    ZG_REQUIRE(L.K > 0 && L.A && L.B && L.C, ZG_ERR_ARG, "linear: empty operand");
-    ZG_REQUIRE(L.a_div >= 1, ZG_ERR_ARG, "linear: a_div %d", L.a_div);
+namespace {
+LinArgs make_args(const Linear& L);
+bool takes_k_split(const Linear& L) { return L.K >= 1536 && L.M <= 2 && L.nz <= 4; }
+}  // namespace
+
+int launch_linear_pair(const Linear& A, const Linear& B, bool f32, hipStream_t s) {
+    const bool one_launch = A.M == 1 && B.M == 1 && A.nz >= 1 && B.nz >= 1 && A.N > 0 && B.N > 0 && !A.grp_off && !B.grp_off && !takes_k_split(A) &&
+                            !takes_k_split(B) && A.K > 0 && B.K > 0 && A.A && A.B && A.C && B.A && B.B && B.C && A.a_div >= 1 && B.a_div >= 1 &&
+                            A.nz + B.nz <= 65535;
+    if (!one_launch) {
+        ZG_TRY(launch_linear(A, f32, s));
+        return launch_linear(B, f32, s);
+    }
+    const dim3 grid((std::max(A.N, B.N) + 7) / 8, 1, A.nz + B.nz);
+    lm_gemv_pair_kernel<<<grid, 256, 0, s>>>(make_args(A), make_args(B), A.nz);
+    note_kernel("lm_gemv_pair_kernel");
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+namespace {
+LinArgs make_args(const Linear& L) {
     LinArgs p;
     p.A = L.A; p.B = L.B; p.C = L.C; p.a_rows = L.a_rows; p.z_group = L.z_group; p.grp_off = L.grp_off;
     p.a_zoff = L.a_zoff; p.b_zoff = L.b_zoff; p.c_zoff = L.c_zoff;
@@ -454,8 +486,17 @@ int launch_linear(const Linear& L, bool f32, hipStream_t s) {
     p.glu_gate_col = L.glu_gate_col;
     p.a_vec = ((reinterpret_cast<uintptr_t>(L.A) & 15) == 0 && L.lda % 4 == 0 && L.a_zoff % 4 == 0) ? 1 : 0;
     p.b_vec = ((reinterpret_cast<uintptr_t>(L.B) & 15) == 0 && L.ldb % 8 == 0 && L.b_zoff % 8 == 0) ? 1 : 0;
+    return p;
+}
+}  // namespace
+
+int launch_linear(const Linear& L, bool f32, hipStream_t s) {
+    if (L.M <= 0 || L.N <= 0 || L.nz <= 0) return ZG_OK;
+    ZG_REQUIRE(L.K > 0 && L.A && L.B && L.C, ZG_ERR_ARG, "linear: empty operand");
+    ZG_REQUIRE(L.a_div >= 1, ZG_ERR_ARG, "linear: a_div %d", L.a_div);
+    const LinArgs p = make_args(L);
     if (!L.grp_off && L.M <= kGemvMaxRows) {
-        if (L.K >= 1536 && L.M <= 2 && L.nz <= 4) {  // long rows, one or two of them, few batches: K split over the waves, two weight rows per workgroup
+        if (takes_k_split(L)) {  // long rows, one or two of them, few batches: K split over the waves, two weight rows per workgroup
             const dim3 gks((L.N + 1) / 2, 1, L.nz);  // (from four rows on the activations are re-read by too many workgroups: measured slower)
             if (L.M == 1) lm_gemv_ks_kernel<1><<<gks, 256, 0, s>>>(p);
             else lm_gemv_ks_kernel<2><<<gks, 256, 0, s>>>(p);

@@ -338,6 +338,83 @@ __global__ __launch_bounds__(256) void norm_plain_kernel(float* v, int ld, int r
     for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i];
 }
 
+// ------------------------------------------------------------------------------------------------ norms without statistics
+// n(v) = tanh(alpha v) * w + b, nw = [w (W) | b (W) | alpha]: elementwise, so a thread takes four neighbours of a row (rows whose
+// width is no multiple of four: one) and every sum around the norm rides in the same pass.
+__device__ __forceinline__ float tanh_norm_f(const float* nw, int W, int i, float alpha, float v) { return fmaf(tanhf(alpha * v), nw[i], nw[W + i]); }
+
+template <int VW>
+__global__ __launch_bounds__(256) void tanh_norm_kernel(float* x, const float* pre, const float* nw, const int* rows, float* out, size_t n, int W) {
+    const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VW;
+    if (idx >= n) return;
+    const size_t j = idx / W;
+    const int i = (int)(idx % W);
+    const size_t src = (rows ? (size_t)rows[j] : j) * W + i;
+    const float ap = pre ? pre[2 * W] : 0.0f, an = nw ? nw[2 * W] : 0.0f;
+    float v[VW];
+    if (VW == 4) {
+        const f32x4 t = *reinterpret_cast<const f32x4*>(x + src);
+        v[0] = t.x; v[VW > 1 ? 1 : 0] = t.y; v[VW > 2 ? 2 : 0] = t.z; v[VW > 3 ? 3 : 0] = t.w;
+    } else {
+        v[0] = x[src];
+    }
+    if (pre) {
+#pragma unroll
+        for (int u = 0; u < VW; ++u) v[u] = tanh_norm_f(pre, W, i + u, ap, v[u]);
+        if (VW == 4) *reinterpret_cast<f32x4*>(x + src) = f32x4{v[0], v[VW > 1 ? 1 : 0], v[VW > 2 ? 2 : 0], v[VW > 3 ? 3 : 0]};
+        else x[src] = v[0];
+    }
+    if (!nw) return;
+#pragma unroll
+    for (int u = 0; u < VW; ++u) v[u] = tanh_norm_f(nw, W, i + u, an, v[u]);
+    if (VW == 4) *reinterpret_cast<f32x4*>(out + idx) = f32x4{v[0], v[VW > 1 ? 1 : 0], v[VW > 2 ? 2 : 0], v[VW > 3 ? 3 : 0]};
+    else out[idx] = v[0];
+}
+
+template <int VW>
+__global__ __launch_bounds__(256) void tanh_sum_norm_kernel(float* x, const SumParts y, const float* nb, float mult, const float* nn, float* h, size_t n,
+                                                            int W) {
+    const size_t idx = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * VW;
+    if (idx >= n) return;
+    const size_t m = idx / W;
+    const int i = (int)(idx % W);
+    auto load = [&](const float* p, float* v) {
+        if (VW == 4) {
+            const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+            v[0] = t.x; v[VW > 1 ? 1 : 0] = t.y; v[VW > 2 ? 2 : 0] = t.z; v[VW > 3 ? 3 : 0] = t.w;
+        } else {
+            v[0] = p[0];
+        }
+    };
+    float a[VW], t[VW], xv[VW];
+#pragma unroll
+    for (int u = 0; u < VW; ++u) a[u] = 0.0f;
+    load(x + idx, xv);
+    if (y.a) load(y.a + idx, a);
+    for (int k = 0; k < y.top; ++k) {  // in choice order: the sum does not depend on the batch
+        const size_t as = m * y.top + k;
+        const float wk = y.exp_w ? y.exp_w[as] : 1.0f;
+        load(y.exp + (size_t)(y.inv ? y.inv[as] : as) * W + i, t);
+#pragma unroll
+        for (int u = 0; u < VW; ++u) a[u] = fmaf(wk, t[u], a[u]);
+    }
+    if (y.b) {
+        load(y.b + idx, t);
+#pragma unroll
+        for (int u = 0; u < VW; ++u) a[u] += t[u];
+    }
+    const float ab = nb[2 * W], an = nn ? nn[2 * W] : 0.0f;
+#pragma unroll
+    for (int u = 0; u < VW; ++u) xv[u] = fmaf(mult, tanh_norm_f(nb, W, i + u, ab, a[u]), xv[u]);
+    if (VW == 4) *reinterpret_cast<f32x4*>(x + idx) = f32x4{xv[0], xv[VW > 1 ? 1 : 0], xv[VW > 2 ? 2 : 0], xv[VW > 3 ? 3 : 0]};
+    else x[idx] = xv[0];
+    if (!nn) return;
+#pragma unroll
+    for (int u = 0; u < VW; ++u) t[u] = tanh_norm_f(nn, W, i + u, an, xv[u]);
+    if (VW == 4) *reinterpret_cast<f32x4*>(h + idx) = f32x4{t[0], t[VW > 1 ? 1 : 0], t[VW > 2 ? 2 : 0], t[VW > 3 ? 3 : 0]};
+    else h[idx] = t[0];
+}
+
 // ------------------------------------------------------------------------------------------------ HGRN2
 // A column j of a head's state S[D][V] is held by G consecutive lanes, 16 rows each (D <= 16 G).  The token loop is serial; the
 // gates and values of the next SB tokens are staged in the LDS (rows beyond D padded with q = 0, f = 1: they stay zero).
@@ -364,19 +441,26 @@ __device__ __forceinline__ bool scan_find_chunk(int id, const int* ent_len, int 
     return false;
 }
 
-// LIN: linear attention with a fixed decay per head on the same layout — the staged "gate" array holds silu(k), the weight of
+// KIND SCAN_LIN: linear attention with a fixed decay per head on the same layout — the staged "gate" array holds silu(k), the weight of
 // the token's value in the state's row, and every row decays by decay[h]:  S <- decay S + k v^T  (q, k, v through silu).
-template <int G, bool LIN>
+// KIND SCAN_GLA: gated linear attention — q (times a factor), k and v unchanged, and one decay per key channel,
+// f = sigmoid(z + bias)^(1 / tau) = exp(log sigmoid(z + bias) / tau) in fp32, staged beside k:  S <- diag(f) S + k v^T.
+enum { SCAN_HGRN2 = 0, SCAN_LIN = 1, SCAN_GLA = 2 };
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.0f) - log1pf(expf(-fabsf(z))); }
+
+template <int G, int KIND>
 __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride,
                                                          const int* ent_start, const int* ent_len, const int* ent_slot, int n_entries, int H, int D,
                                                          int V, int mode, int SB, float* wsB, float* wsA, const float* bias, const float* low,
-                                                         const float* decay) {
+                                                         const float* decay, const GlaGate gla) {
+    constexpr bool LIN = KIND == SCAN_LIN, GLA = KIND == SCAN_GLA;
     extern __shared__ __attribute__((aligned(16))) float s_scan[];
     constexpr int Dp = G * kScanRows;
     const int cols = blockDim.x / G;
     float* sq = s_scan;             // [SB][Dp]
     float* sf = sq + SB * Dp;       // [SB][Dp]
     float* sv = sf + SB * Dp;       // [SB][cols]
+    float* sk = sv + SB * cols;     // [SB][Dp] (SCAN_GLA: the keys; the gate array holds the decays)
     const int h = blockIdx.y;
     const int jl = threadIdx.x / G, g = threadIdx.x % G, j0 = blockIdx.z * cols, j = j0 + jl;
     const bool col_ok = j < V;
@@ -411,18 +495,25 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
             const int tt = idx / Dp, i = idx % Dp;
             const float* row = proj + (size_t)(m0 + tb + tt) * ld;
             // the gates are activated on their way into the LDS: q = silu(.), f = low + (1 - low) sigmoid(. + bias)
-            float qv = 0.0f, fv = LIN ? 0.0f : 1.0f;
+            float qv = 0.0f, fv = LIN ? 0.0f : 1.0f, kv = 0.0f;
             if (i < D) {
-                qv = silu_f(row[h * D + i]);
-                if (LIN) {
-                    fv = silu_f(row[HD + h * D + i]);
+                if (GLA) {
+                    qv = row[h * D + i] * gla.q_scale;
+                    kv = row[HD + h * D + i];
+                    fv = expf(log_sigmoid_f(gla.z[(size_t)(m0 + tb + tt) * gla.ldz + h * D + i] + gla.z_bias[h * D + i]) * gla.inv_tau);
                 } else {
-                    const float l = low[h * D + i];
-                    fv = l + (1.0f - l) * sigmoid_f(row[HD + h * D + i] + bias[h * D + i]);
+                    qv = silu_f(row[h * D + i]);
+                    if (LIN) {
+                        fv = silu_f(row[HD + h * D + i]);
+                    } else {
+                        const float l = low[h * D + i];
+                        fv = l + (1.0f - l) * sigmoid_f(row[HD + h * D + i] + bias[h * D + i]);
+                    }
                 }
             }
             sq[idx] = qv;
             sf[idx] = fv;
+            if (GLA) sk[idx] = kv;
         }
         for (int idx = threadIdx.x; idx < nb * cols; idx += blockDim.x) {
             const int tt = idx / cols, jj = idx % cols;
@@ -433,16 +524,18 @@ __global__ __launch_bounds__(256) void hgrn2_scan_kernel(const float* proj, int 
         for (int tt = 0; tt < nb; ++tt) {
             const f32x4* q4 = reinterpret_cast<const f32x4*>(sq + tt * Dp + g * kScanRows);
             const f32x4* f4 = reinterpret_cast<const f32x4*>(sf + tt * Dp + g * kScanRows);
+            const f32x4* k4 = reinterpret_cast<const f32x4*>(sk + tt * Dp + g * kScanRows);
             const float v = sv[tt * cols + jl];
             float o = 0.0f;
 #pragma unroll
             for (int r4 = 0; r4 < kScanRows / 4; ++r4) {
                 const f32x4 qq = q4[r4], ff = f4[r4];
-                const float qv[4] = {qq.x, qq.y, qq.z, qq.w}, fv[4] = {ff.x, ff.y, ff.z, ff.w};
+                const f32x4 kk = GLA ? k4[r4] : ff;
+                const float qv[4] = {qq.x, qq.y, qq.z, qq.w}, fv[4] = {ff.x, ff.y, ff.z, ff.w}, kv[4] = {kk.x, kk.y, kk.z, kk.w};
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int r = r4 * 4 + u;
-                    S[r] = LIN ? fmaf(dec, S[r], fv[u] * v) : fmaf(fv[u], S[r], (1.0f - fv[u]) * v);
+                    S[r] = GLA ? fmaf(fv[u], S[r], kv[u] * v) : LIN ? fmaf(dec, S[r], fv[u] * v) : fmaf(fv[u], S[r], (1.0f - fv[u]) * v);
                     o = fmaf(S[r], qv[u], o);
                     if (mode == SCAN_A) A[r] *= LIN ? dec : fv[u];
                 }
@@ -1137,6 +1230,29 @@ int launch_add_two(float* x, const OpenSums& add, int M, int W, hipStream_t s) {
     return ZG_OK;
 }
 
+int launch_tanh_norm(float* x, const float* pre, const float* nw, const int* rows, float* out, int n_rows, int W, hipStream_t s) {
+    const size_t n = (size_t)n_rows * W;
+    if (n == 0) return ZG_OK;
+    ZG_REQUIRE((pre || nw) && (!nw || out) && !(pre && rows), ZG_ERR_ARG, "tanh norm: nothing to do, no output, or an in-place norm of gathered rows");
+    const bool vec = W % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) & 15) == 0;
+    if (vec) tanh_norm_kernel<4><<<(unsigned)((n / 4 + 255) / 256), 256, 0, s>>>(x, pre, nw, rows, out, n, W);
+    else tanh_norm_kernel<1><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, pre, nw, rows, out, n, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_tanh_sum_norm(float* x, const SumParts& y, const float* nb, float mult, const float* nn, float* h, int M, int W, hipStream_t s) {
+    const size_t n = (size_t)M * W;
+    if (n == 0) return ZG_OK;
+    ZG_REQUIRE(nb && (!nn || h) && (y.top == 0 || y.exp), ZG_ERR_ARG, "tanh norm behind a sum: no norm, no output, or no rows of the experts");
+    const uintptr_t al = reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(y.a) |
+                         reinterpret_cast<uintptr_t>(y.exp) | reinterpret_cast<uintptr_t>(y.b);
+    if (W % 4 == 0 && (al & 15) == 0) tanh_sum_norm_kernel<4><<<(unsigned)((n / 4 + 255) / 256), 256, 0, s>>>(x, y, nb, mult, nn, h, n, W);
+    else tanh_sum_norm_kernel<1><<<(unsigned)((n + 255) / 256), 256, 0, s>>>(x, y, nb, mult, nn, h, n, W);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
 int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, hipStream_t s) {
     const int n_vec = M * rows_per_m;
     if (n_vec <= 0) return ZG_OK;
@@ -1147,8 +1263,10 @@ int launch_norm_plain(float* v, int ld, int rows_per_m, int width, int M, const 
 
 int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* state, size_t slot_stride, const int* ent_start,
                       const int* ent_len, const int* ent_slot, int n_entries, int M, int H, int D, int V, const float* bias, const float* low,
-                      float* ws, size_t ws_floats, hipStream_t s, const float* decay) {
+                      float* ws, size_t ws_floats, hipStream_t s, const float* decay, const GlaGate* gla) {
     if (n_entries <= 0) return ZG_OK;
+    ZG_REQUIRE(!gla || (gla->z && gla->z_bias && !decay), ZG_ERR_ARG, "gated linear attention: its gate needs z and a bias, and no fixed decay");
+    const GlaGate gg = gla ? *gla : GlaGate();
     ZG_REQUIRE(D >= 1 && D <= 16 * kScanRows, ZG_ERR_UNSUPPORTED, "hgrn2: %d key channels per head (at most %d)", D, 16 * kScanRows);
     if (decay && M > kGemvMaxRows && D <= 128 && ws && getenv("ZGPT2_LM_LINEAR_NO_CHUNKS") == nullptr) {
         // a scalar decay per head: chunks of kLinChunk tokens as matrix products (prompt portions; the test hook sends them through the scan)
@@ -1179,22 +1297,23 @@ int launch_hgrn2_scan(const float* proj, int ld, float* out, int ldo, float* sta
     int threads = ((V * G + 63) / 64) * 64;
     if (threads > 256) threads = 256;
     const int cols = threads / G;
-    const int SB = std::max(1, std::min(kScanChunk, std::min(4096 / Dp, 8192 / cols)));
-    const size_t lds = ((size_t)2 * SB * Dp + (size_t)SB * cols) * sizeof(float);
+    const int SB = std::max(1, std::min(kScanChunk, std::min((gla ? 2560 : 4096) / Dp, 8192 / cols)));
+    const size_t lds = ((size_t)(gla ? 3 : 2) * SB * Dp + (size_t)SB * cols) * sizeof(float);
     // chunked when the step is long enough to pay for two passes, and the workspace holds every chunk's state
     const int max_chunks = (M + kScanChunk - 1) / kScanChunk + n_entries;
     const size_t head_floats = (size_t)H * D * V, need = (size_t)max_chunks * (head_floats + (size_t)H * D);
     const bool chunked = M >= 4 * kScanChunk && ws && ws_floats >= need;
     float* wsB = chunked ? ws : nullptr;
     float* wsA = chunked ? ws + (size_t)max_chunks * head_floats : nullptr;
-#define ZG_SCAN_L(G_, LIN_, grid_x, mode)                                                                                                   \
-    hgrn2_scan_kernel<G_, LIN_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start,     \
-                                                                                              ent_len, ent_slot, n_entries, H, D, V, mode, SB, wsB, \
-                                                                                              wsA, bias, low, decay)
-#define ZG_SCAN(G_, grid_x, mode)                    \
-    do {                                             \
-        if (decay) ZG_SCAN_L(G_, true, grid_x, mode); \
-        else ZG_SCAN_L(G_, false, grid_x, mode);     \
+#define ZG_SCAN_L(G_, KIND_, grid_x, mode)                                                                                                  \
+    hgrn2_scan_kernel<G_, KIND_><<<dim3(grid_x, H, (V + cols - 1) / cols), threads, lds, s>>>(proj, ld, out, ldo, state, slot_stride, ent_start,    \
+                                                                                               ent_len, ent_slot, n_entries, H, D, V, mode, SB, wsB, \
+                                                                                               wsA, bias, low, decay, gg)
+#define ZG_SCAN(G_, grid_x, mode)                         \
+    do {                                                  \
+        if (gla) ZG_SCAN_L(G_, SCAN_GLA, grid_x, mode);   \
+        else if (decay) ZG_SCAN_L(G_, SCAN_LIN, grid_x, mode); \
+        else ZG_SCAN_L(G_, SCAN_HGRN2, grid_x, mode);     \
     } while (0)
 #define ZG_SCAN_G(grid_x, mode)                    \
     switch (G) {                                   \

@@ -28,14 +28,41 @@ __device__ __forceinline__ float block_allsum(float v, float* s_red) {
 // logits meet in the LDS and wave 0 does the softmax and the choice, lane e % 64 holding expert e (four slots per lane).
 // top_logits: the correction is a bias of the logits, the largest logits are chosen and the weights are the softmax over the chosen
 // logits alone.
+// sigmoid scores with groups: experts ranked by r = sigmoid(z) + correction; a block of adjacent experts ranks by its best r plus
+// its second-best r, only the `keep` top-ranked blocks (lowest index wins a tie) remain eligible; the weights are the winners'
+// sigmoid(z) over their sum, times out_scale.
+// pre.x != null: the workgroup first finishes its own row — x += mult * nb(sum of the sublayer's parts), h = nn(x), both written
+// out, h also kept in the LDS — and routes on that (steps of few rows: the sum and norm in front of the router need no launch
+// of their own).
 __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top,
-                                                    int* pick, float* weight, int rule) {
-    const bool top_logits = rule != 0;  // rules that choose by the logits themselves
+                                                    int* pick, float* weight, int rule, int groups, int keep, float out_scale, const RoutePre pre) {
+    const bool top_logits = rule == 1 || rule == 2;  // rules that choose by the logits themselves
     const bool sigmoid_w = rule == 2;   // ... and weigh a chosen expert by sigmoid(z), nothing renormalised
+    extern __shared__ __attribute__((aligned(16))) float s_row[];  // [W] with pre
     __shared__ float s_z[kMaxExperts];
+    __shared__ float s_gs[kMaxExperts];
     const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* row = g + (size_t)m * W;
-    const bool vec = (W % 8 == 0) && ((reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(router) & 15) == 0);
+    if (pre.x) {
+        const float ab = pre.nb[2 * W], an = pre.nn[2 * W];
+        for (int i = threadIdx.x; i < W; i += blockDim.x) {
+            const size_t idx = (size_t)m * W + i;
+            float a = pre.y.a ? pre.y.a[idx] : 0.0f;
+            for (int k = 0; k < pre.y.top; ++k) {
+                const size_t as = (size_t)m * pre.y.top + k;
+                a = fmaf(pre.y.exp_w ? pre.y.exp_w[as] : 1.0f, pre.y.exp[(size_t)(pre.y.inv ? pre.y.inv[as] : as) * W + i], a);
+            }
+            if (pre.y.b) a += pre.y.b[idx];
+            const float v = fmaf(pre.mult, fmaf(tanhf(ab * a), pre.nb[i], pre.nb[W + i]), pre.x[idx]);
+            const float hv = fmaf(tanhf(an * v), pre.nn[i], pre.nn[W + i]);
+            pre.x[idx] = v;
+            pre.h[idx] = hv;
+            s_row[i] = hv;
+        }
+        __syncthreads();
+        row = s_row;
+    }
+    const bool vec = (W % 8 == 0) && (pre.x || (reinterpret_cast<uintptr_t>(g) & 15) == 0) && ((reinterpret_cast<uintptr_t>(router) & 15) == 0);
     for (int e = wave; e < E; e += 4) {
         const bf16_t* wr = router + (size_t)e * W;
         float a = 0.0f;
@@ -70,6 +97,26 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
         if (lane == 0) s_z[e] = a;
     }
     __syncthreads();
+    if (rule == 3 && groups > 1) {  // every block's rank, by all four waves: its best r plus its second-best r
+        __shared__ float s_c[kMaxExperts];
+        const int gsz = E / groups;
+        for (int e = threadIdx.x; e < E; e += blockDim.x) s_c[e] = 1.0f / (1.0f + expf(-s_z[e])) + (correction ? correction[e] : 0.0f);
+        __syncthreads();
+        for (int gi = threadIdx.x; gi < groups; gi += blockDim.x) {
+            float a = -INFINITY, b = -INFINITY;
+            for (int e = gi * gsz; e < (gi + 1) * gsz; ++e) {
+                const float c = s_c[e];
+                if (c > a) {
+                    b = a;
+                    a = c;
+                } else if (c > b) {
+                    b = c;
+                }
+            }
+            s_gs[gi] = gsz > 1 ? a + b : a;
+        }
+        __syncthreads();
+    }
     if (wave != 0) return;
     float z[4], sc[4], ch[4];
 #pragma unroll
@@ -114,6 +161,60 @@ __global__ __launch_bounds__(256) void route_kernel(const float* g, int M, int W
 #pragma unroll
         for (int i = 0; i < 4; ++i)
             if (lane + 64 * i < top) weight[(size_t)m * top + lane + 64 * i] = ek[i] / sum;
+        return;
+    }
+    if (rule == 3) {
+        int pk[4] = {0, 0, 0, 0};  // 1 + the place of the expert among the chosen
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = lane + 64 * i;
+            sc[i] = e < E ? 1.0f / (1.0f + expf(-z[i])) : 0.0f;
+            ch[i] = e < E ? sc[i] + (correction ? correction[e] : 0.0f) : -INFINITY;
+        }
+        if (groups > 1) {
+            const int gsz = E / groups;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int e = lane + 64 * i;
+                if (e >= E) continue;
+                const int mine = e / gsz;
+                const float ms = s_gs[mine];
+                int ahead = 0;  // groups that come before this expert's group
+                for (int o = 0; o < groups; ++o) ahead += (s_gs[o] > ms || (s_gs[o] == ms && o < mine)) ? 1 : 0;
+                if (ahead >= keep) ch[i] = -INFINITY;
+            }
+        }
+        for (int k = 0; k < top; ++k) {
+            float best = -INFINITY;
+            int bi = 0x7fffffff;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (ch[i] > best) {  // ascending expert index per lane: the first maximum stays
+                    best = ch[i];
+                    bi = lane + 64 * i;
+                }
+            const float wbest = wave_allmax(best);
+            int cand = (best == wbest) ? bi : 0x7fffffff;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) cand = min(cand, __shfl_xor(cand, off, 64));
+            if (cand == 0x7fffffff) cand = 0;  // nothing left to choose from: keep the indices in range
+            if ((cand & 63) == lane) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if ((cand >> 6) == i) {
+                        pick[(size_t)m * top + k] = cand;
+                        pk[i] = k + 1;
+                        ch[i] = -INFINITY;
+                    }
+            }
+        }
+        float mine = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mine += pk[i] ? sc[i] : 0.0f;
+        const float total = wave_allsum(mine) + 1e-20f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (pk[i]) weight[(size_t)m * top + pk[i] - 1] = sc[i] / total * out_scale;
         return;
     }
     const float mx = wave_allmax(fmaxf(fmaxf(z[0], z[1]), fmaxf(z[2], z[3])));
@@ -252,11 +353,18 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* x, const float*
 }  // namespace
 
 int launch_route(const float* g, int M, int W, const bf16_t* router, const float* correction, int E, int top, int* pick, float* weight,
-                 int rule, hipStream_t s) {
+                 int rule, hipStream_t s, int groups, int keep, float out_scale, const RoutePre* pre) {
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(E >= 1 && E <= kMaxExperts && top >= 1 && top <= E, ZG_ERR_UNSUPPORTED, "router: %d experts, %d chosen (at most %d experts)", E, top,
                kMaxExperts);
-    route_kernel<<<M, 256, 0, s>>>(g, M, W, router, correction, E, top, pick, weight, rule);
+    if (groups < 1) groups = 1;
+    if (keep < 1) keep = groups;  // (a descriptor that names no groups)
+    ZG_REQUIRE(E % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (E / groups), ZG_ERR_ARG,
+               "router: %d experts in %d groups, %d groups kept, %d chosen", E, groups, keep, top);
+    ZG_REQUIRE(!pre || (pre->x && pre->nb && pre->nn && pre->h == g && W <= kRouteFuseWidth), ZG_ERR_ARG,
+               "router: the sum in front of it needs x, both norms, its output as the router's input, and a width of at most %d", kRouteFuseWidth);
+    route_kernel<<<M, 256, pre ? (size_t)W * sizeof(float) : 0, s>>>(g, M, W, router, correction, E, top, pick, weight, rule, groups, keep, out_scale,
+                                                                     pre ? *pre : RoutePre());
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

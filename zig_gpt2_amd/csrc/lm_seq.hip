@@ -260,6 +260,13 @@ __device__ __forceinline__ KeySpan key_span(int pos, int window, int keep) {
 }
 __device__ __forceinline__ int key_pos(const KeySpan& k, int n) { return n < k.n_first ? n : k.j_lo + (n - k.n_first); }
 
+// a scaled score on its way to the softmax: capped, then less the head's slope per position of distance (fp32)
+__device__ __forceinline__ float shape_score(float sc, const ScoreShape& sh, int h, int dist) {
+    if (sh.cap > 0.0f) sc = sh.cap * tanhf(sc / sh.cap);
+    if (sh.slope) sc -= sh.slope[h] * (float)dist;
+    return sc;
+}
+
 constexpr int kWinTile = 64;
 constexpr int kWinMaxHeads = 64;
 constexpr int kWinAcc = 16;  // outputs per thread: H * V <= 256 * kWinAcc
@@ -267,7 +274,8 @@ constexpr int kWinAcc = 16;  // outputs per thread: H * V <= 256 * kWinAcc
 __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, int ldq, float* out, int ldo, int H, int G, int D, int V,
                                                                float scale, int window, int keep, const float* sink, const float* talk,
                                                                const float* vfreq, const int* row_pos, const int* row_slot,
-                                                               const int* page_table, int max_pages, int page_tokens, const float* cache) {
+                                                               const int* page_table, int max_pages, int page_tokens, const float* cache,
+                                                               const ScoreShape shape) {
     extern __shared__ __attribute__((aligned(16))) float s_win[];
     float* s_q = s_win;                       // [H D]
     float* s_s = s_q + H * D;                 // [H][kWinTile] scores, then weights
@@ -308,7 +316,7 @@ __global__ __launch_bounds__(256) void window_attention_kernel(const float* q, i
                 const float* qh = s_q + h * D;
                 float a = 0.0f;
                 for (int d = 0; d < D; ++d) a = fmaf(qh[d], kr[d], a);
-                s = a * scale;
+                s = shape_score(a * scale, shape, h, pos - key_pos(span, t0 + jj));
             }
             s_s[idx] = s;
         }
@@ -400,7 +408,8 @@ constexpr int kScoreKeys = 8;    // keys a wave has in flight
 template <int RPL>
 __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
                                                             int keep, const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
-                                                            int page_tokens, const float* cache, float* sc, int NK, float* st) {
+                                                            int page_tokens, const float* cache, float* sc, int NK, float* st,
+                                                            const ScoreShape shape) {
     extern __shared__ __attribute__((aligned(16))) float s_sc[];
     float* s_q = s_sc;                     // [H][64 RPL] (zero beyond D)
     float* s_t = s_q + H * 64 * RPL;       // [H][kScoreTile] scores of the tile
@@ -456,6 +465,7 @@ __global__ __launch_bounds__(256) void window_scores_kernel(const float* q, int 
                         float mine = a[0];
 #pragma unroll
                         for (int u = 1; u < kScoreKeys; ++u) mine = lane == u ? a[u] : mine;
+                        mine = shape_score(mine, shape, h, pos - key_pos(span, t0 + kk + lane));
                         s_t[h * kScoreTile + kk + lane] = mine;
                         srow[(size_t)h * NK + t0 + kk + lane] = mine;
                     }
@@ -507,7 +517,7 @@ template <int DH>
 __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q, int ldq, int H, int G, int D, int V, float scale, int window,
                                                                  int keep, const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
                                                                  const int* row_slot, const int* page_table, int max_pages, int page_tokens,
-                                                                 const float* cache, float* sc, int NK) {
+                                                                 const float* cache, float* sc, int NK, const ScoreShape shape) {
     int e, b;
     if (!rows_find_block(blockIdx.x, ent_len, n_entries, e, b)) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, kh = lane >> 5;
@@ -567,7 +577,7 @@ __global__ __launch_bounds__(256) void window_scores_mfma_kernel(const float* q,
                 const int pi = pos0 + qi;
                 const KeySpan sp = key_span(pi, window, keep);
                 if (qi < nrows && j <= pi && (j >= sp.j_lo || j < sp.n_first))
-                    sc[((size_t)(m0 + qi) * H + h) * NK + (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j)] = acc[i] * scale;
+                    sc[((size_t)(m0 + qi) * H + h) * NK + (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j)] = shape_score(acc[i] * scale, shape, h, pi - j);
             }
         }
     }
@@ -1055,26 +1065,26 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(const float* qk, int ld
 
 // one wave per (row, head) vector, in place: v / rms(v) * w * sigmoid(gate)
 __global__ __launch_bounds__(256) void norm_gate_kernel(float* v, int ld, int rows_per_m, int width, int n_vec, const float* w, float eps,
-                                                        const float* gate, int ldg, float factor) {
+                                                        const float* gate, int ldg, float factor, bool gate_silu) {
     const int vec = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (vec >= n_vec) return;
     const size_t m = vec / rows_per_m, hh = vec % rows_per_m;
     float* p = v + m * ld + hh * width;
     const float* gp = gate + m * ldg + hh * width;
     if (!w) {  // the gate and the factor only
-        for (int i = lane; i < width; i += 64) p[i] = p[i] * sigmoid_f(gp[i]) * factor;
+        for (int i = lane; i < width; i += 64) p[i] = p[i] * sigmoid_f(gp[i]) * (gate_silu ? gp[i] : 1.0f) * factor;
         return;
     }
     float ss = 0.0f;
     for (int i = lane; i < width; i += 64) ss = fmaf(p[i], p[i], ss);
     ss = wave_allsum(ss);
     const float r = 1.0f / sqrtf(ss / (float)width + eps) * factor;
-    for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i] * sigmoid_f(gp[i]);
+    for (int i = lane; i < width; i += 64) p[i] = p[i] * r * w[i] * sigmoid_f(gp[i]) * (gate_silu ? gp[i] : 1.0f);
 }
 
 // the same for wide vectors: a workgroup per vector
 __global__ __launch_bounds__(256) void norm_gate_wide_kernel(float* v, int ld, int rows_per_m, int width, const float* w, float eps, const float* gate,
-                                                             int ldg, float factor) {
+                                                             int ldg, float factor, bool gate_silu) {
     __shared__ float s_red[8];
     const size_t m = blockIdx.x / rows_per_m, hh = blockIdx.x % rows_per_m;
     float* p = v + m * ld + hh * width;
@@ -1086,7 +1096,7 @@ __global__ __launch_bounds__(256) void norm_gate_wide_kernel(float* v, int ld, i
         ss = block_allsum(ss, s_red);
         r = 1.0f / sqrtf(ss / (float)width + eps) * factor;
     }
-    for (int i = threadIdx.x; i < width; i += blockDim.x) p[i] = p[i] * r * (w ? w[i] : 1.0f) * sigmoid_f(gp[i]);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) p[i] = p[i] * r * (w ? w[i] : 1.0f) * sigmoid_f(gp[i]) * (gate_silu ? gp[i] : 1.0f);
 }
 
 // Decode steps (one row per entry) of the attention below: biases, the short convolutions of q | k | v with their tails moved
@@ -1181,6 +1191,35 @@ __global__ __launch_bounds__(256) void whole_norm_prep_kernel(float* qkv, int ld
     for (int i = threadIdx.x; i < GV; i += blockDim.x) crow[GD + i] = v[i];
 }
 
+// Attention whose q and k are divided by their root mean square per head, and whose values reuse its un-normalised key projection: one
+// workgroup per row, a wave per head (query heads, then key heads).  The query's factor grows with the logarithm of its position;
+// the cache row receives the normed key heads and, behind them, the projected ones.
+__global__ __launch_bounds__(256) void head_norm_prep_kernel(float* qk, int ld, int H, int G, int D, float eps, float qt_coef, int qt_every,
+                                                             const int* row_pos, const int* row_slot, const int* page_table, int max_pages,
+                                                             int page_tokens, float* cache) {
+    const int m = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int pos = row_pos[m];
+    const int page = page_table[(size_t)row_slot[m] * max_pages + (pos / page_tokens) % max_pages];
+    float* crow = cache + ((size_t)page * page_tokens + pos % page_tokens) * ((size_t)2 * G * D);
+    const float qf = qt_every > 0 ? 1.0f + qt_coef * logf((float)((pos + 1) / qt_every + 1)) : 1.0f;
+    for (int u = wave; u < H + G; u += 4) {
+        float* p = qk + (size_t)m * ld + (size_t)u * D;
+        float ss = 0.0f;
+        for (int i = lane; i < D; i += 64) ss = fmaf(p[i], p[i], ss);
+        ss = wave_allsum(ss);
+        const float r = 1.0f / sqrtf(ss / (float)D + eps);
+        if (u < H) {
+            for (int i = lane; i < D; i += 64) p[i] = p[i] * r * qf;
+        } else {
+            const int g = u - H;
+            for (int i = lane; i < D; i += 64) {
+                crow[(size_t)g * D + i] = p[i] * r;
+                crow[(size_t)(G + g) * D + i] = p[i];
+            }
+        }
+    }
+}
+
 }  // namespace
 
 int launch_add_rows(float* x, const float* y, int M, int W, hipStream_t s) {
@@ -1250,7 +1289,7 @@ int launch_whole_norm_prep(float* qkv, int ld, int M, int HD, int GD, int GV, co
 
 int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M, int H, int G, int D, int V, float scale, int window,
                             int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
-                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s) {
+                            const int* page_table, int max_pages, int page_tokens, const float* cache, hipStream_t s, ScoreShape shape) {
     if (M <= 0) return ZG_OK;
     ZG_REQUIRE(H >= 1 && H <= kWinMaxHeads && G >= 1 && H % G == 0, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads on %d key heads (at most %d heads)",
                H, G, kWinMaxHeads);
@@ -1259,7 +1298,17 @@ int launch_window_attention(const float* q, int ldq, float* out, int ldo, int M,
     const size_t lds = ((size_t)H * D + 2 * (size_t)H * kWinTile + (size_t)H * H + (size_t)H * V) * sizeof(float);
     ZG_REQUIRE(lds <= 60 * 1024, ZG_ERR_UNSUPPORTED, "windowed attention: %d heads of %d + %d channels need %zu bytes of LDS", H, D, V, lds);
     window_attention_kernel<<<M, 256, lds, s>>>(q, ldq, out, ldo, H, G, D, V, scale, window, window > 0 ? keep_first : 0, sink, talk, vfreq, row_pos, row_slot, page_table,
-                                                max_pages, page_tokens, cache);
+                                                max_pages, page_tokens, cache, shape);
+    ZG_HIP(hipGetLastError());
+    return ZG_OK;
+}
+
+int launch_head_norm_prep(float* qk, int ld, int M, int H, int G, int D, float eps, float qt_coef, int qt_every, const int* row_pos,
+                          const int* row_slot, const int* page_table, int max_pages, int page_tokens, float* cache, hipStream_t s) {
+    if (M <= 0) return ZG_OK;
+    ZG_REQUIRE(H >= 1 && G >= 1 && D >= 1 && ld >= (H + G) * D && qt_every >= 0, ZG_ERR_ARG, "attention prep: %d + %d heads of %d channels in rows of %d", H,
+               G, D, ld);
+    head_norm_prep_kernel<<<M, 256, 0, s>>>(qk, ld, H, G, D, eps, qt_coef, qt_every, row_pos, row_slot, page_table, max_pages, page_tokens, cache);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }
@@ -1275,7 +1324,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
                                   int keep_first, const float* sink, const float* talk, const float* vfreq, const int* row_pos, const int* row_slot,
                                   const int* page_table, int max_pages, int page_tokens, const float* cache, int key_capacity, float* ws,
                                   size_t ws_floats, const int* ent_start, const int* ent_len, int n_entries, hipStream_t s, bool* taken,
-                                  const float* out_gate, int ld_gate, float out_factor) {
+                                  const float* out_gate, int ld_gate, float out_factor, ScoreShape shape) {
     *taken = false;
     if (M <= 0) return ZG_OK;
     const int keep = window > 0 ? keep_first : 0;
@@ -1304,7 +1353,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
         const dim3 tg((M + 31) / 32 + n_entries, ksplit);
 #define ZG_WT(R)                                                                                                                                   \
     window_scores_mfma_kernel<R><<<tg, 256, 0, s>>>(q, ldq, H, G, D, V, scale, window, keep, ent_start, ent_len, n_entries, row_pos, row_slot, page_table, \
-                                                    max_pages, page_tokens, cache, sc, key_capacity)
+                                                    max_pages, page_tokens, cache, sc, key_capacity, shape)
         if (dh <= 8) ZG_WT(8);
         else if (dh <= 16) ZG_WT(16);
         else if (dh <= 32) ZG_WT(32);
@@ -1316,7 +1365,7 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
     } else {
 #define ZG_WS(R)                                                                                                                              \
     window_scores_kernel<R><<<grid, 256, lds_a, s>>>(q, ldq, H, G, D, V, scale, window, keep, row_pos, row_slot, page_table, max_pages, page_tokens, cache, \
-                                                     sc, key_capacity, st)
+                                                     sc, key_capacity, st, shape)
     if (rpl <= 1) ZG_WS(1);
     else if (rpl <= 2) ZG_WS(2);
     else ZG_WS(4);
@@ -1389,15 +1438,15 @@ int launch_delta_scan(const float* qk, int ldqk, const float* v, int ldv, const 
 }
 
 int launch_norm_gate(float* v, int ld, int rows_per_m, int width, int M, const float* w, float eps, const float* gate, int ldg, hipStream_t s,
-                     float factor) {
+                     float factor, bool gate_silu) {
     const int n_vec = M * rows_per_m;
     if (n_vec <= 0) return ZG_OK;
     if (width > 256) {  // a workgroup per vector
-        norm_gate_wide_kernel<<<n_vec, 256, 0, s>>>(v, ld, rows_per_m, width, w, eps, gate, ldg, factor);
+        norm_gate_wide_kernel<<<n_vec, 256, 0, s>>>(v, ld, rows_per_m, width, w, eps, gate, ldg, factor, gate_silu);
         ZG_HIP(hipGetLastError());
         return ZG_OK;
     }
-    norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg, factor);
+    norm_gate_kernel<<<(n_vec + 3) / 4, 256, 0, s>>>(v, ld, rows_per_m, width, n_vec, w, eps, gate, ldg, factor, gate_silu);
     ZG_HIP(hipGetLastError());
     return ZG_OK;
 }

@@ -160,9 +160,15 @@ typedef std::vector<std::pair<std::string, std::vector<float>>> DerivedTensors;
 inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm_layer>& layers, zg_lm_config& out, DerivedTensors* derived = nullptr) {
     const Json* arch = cfg.get("architecture");
     const std::string design = arch ? arch->str : std::string("?");
-    if (design != "Tokosun" && design != "Gupizen" && design != "Sanazen") throw std::runtime_error("config: architecture '" + design + "' is not served");
-    const bool gup = design == "Gupizen", san = design == "Sanazen";
+    if (design != "Tokosun" && design != "Gupizen" && design != "Sanazen" && design != "Vovalorn")
+        throw std::runtime_error("config: architecture '" + design + "' is not served");
+    const bool gup = design == "Gupizen", san = design == "Sanazen", vov = design == "Vovalorn";
     memset(&out, 0, sizeof(out));
+    if (vov) {  // what the name fixes: norms without statistics, one of them behind the embedding
+        out.flags |= ZG_LM_TANH_NORMS | ZG_LM_EMBED_NORM;
+        out.residual_mult = 1.0f;
+        if (const Json* v = cfg.get("residual_mult")) out.residual_mult = (float)v->num;
+    }
     if (san) {  // what the name fixes: side-by-side sublayers with plain norms, sinusoid positions
         out.flags |= ZG_LM_SIDE_BY_SIDE | ZG_LM_SINUSOID_POSITIONS;
         out.embed_scale = 1.0f;
@@ -195,16 +201,29 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
             out.loop_stop = (int)loop->at("stop").num;
             out.loop_times = (int)loop->at("times").num;
         }
-    for (const Json& e : cfg.at("layers").arr) {
+    const std::vector<Json>& entries = cfg.at("layers").arr;
+    auto owner = [&](size_t i) {  // the layer whose tensors layer i runs
+        for (size_t hops = 0; hops <= entries.size(); ++hops) {
+            const Json* w = entries.at(i).get("weights_of");
+            if (!w || w->kind != Json::Num) return i;
+            if (w->num < 0 || (size_t)w->num >= entries.size()) break;
+            i = (size_t)w->num;
+        }
+        throw std::runtime_error("config: a layer's weights_of names no layer with tensors");
+    };
+    for (const Json& e : entries) {
         zg_lm_layer d;
         memset(&d, 0, sizeof(d));
         const std::string& type = e.at("type").str;
         const Json& m = e.at("mixer");
-        const std::string prefix = "l" + std::to_string(layer_index++) + ".";
+        const size_t own = owner(layer_index);
+        if (own != layer_index) d.weights_of = (int)own + 1;
+        ++layer_index;
+        const std::string prefix = "l" + std::to_string(own) + ".";
         const Json& sizes = ((gup || san) && type == "parallel") ? m.at("left") : m;
         d.heads = (int)sizes.at("heads").num;
         d.dim = (int)sizes.at("dim").num;
-        d.vdim = (int)sizes.at("vdim").num;
+        d.vdim = sizes.get("vdim") ? (int)sizes.at("vdim").num : d.dim;
         if (gup) {
             d.ff_act = ZG_LM_ACT_GELU;
             d.router = ZG_LM_ROUTE_TOP_LOGITS;
@@ -275,6 +294,35 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
             d.gate_rank = inner("gate_rank", "mix.g1");
         } else if (gup) {
             throw std::runtime_error("config: unknown mixer type '" + type + "'");
+        } else if (vov && type == "gla") {
+            d.mixer = ZG_LM_MIX_GLA;
+            d.ff_act = ZG_LM_ACT_GLU_SILU;
+            d.router = ZG_LM_ROUTE_SIGMOID_GROUPS;
+            d.tau = (float)m.at("tau").num;
+            if (const Json* v = m.get("decay_rank")) {
+                d.decay_rank = (int)v->num;
+            } else {
+                const Json* t = tensors ? tensors->get(prefix + "mix.a1") : nullptr;
+                if (!t) throw std::runtime_error("config: the inner size 'decay_rank' needs the shape of tensor " + prefix + "mix.a1");
+                d.decay_rank = (int)t->at("shape").arr.at(0).num;
+            }
+        } else if (vov && type == "attention") {
+            d.mixer = ZG_LM_MIX_ATTENTION;
+            d.ff_act = ZG_LM_ACT_GLU_SILU;
+            d.router = ZG_LM_ROUTE_SIGMOID_GROUPS;
+            d.kv_heads = m.get("kv_heads") ? (int)m.at("kv_heads").num : d.heads;
+            d.scale = (float)m.at("scale").num;
+            if (const Json* v = m.get("softcap"))
+                if (v->truthy()) d.softcap = (float)v->num;
+            if (const Json* qt = m.get("q_temp"))
+                if (qt->truthy()) {
+                    d.qtemp_coef = (float)qt->at("coef").num;
+                    d.qtemp_every = (int)qt->at("every").num;
+                }
+            d.dist_bias = 1;
+            if (const Json* v = m.get("dist_bias")) d.dist_bias = v->truthy() ? 1 : 0;
+        } else if (vov) {
+            throw std::runtime_error("config: unknown mixer type '" + type + "'");
         } else if (type == "hgrn2") {
             d.mixer = ZG_LM_MIX_HGRN2;
         } else if (type == "latent_attention") {
@@ -319,6 +367,18 @@ inline void build_config(const Json& cfg, const Json* tensors, std::vector<zg_lm
                         d.shared_width = (int)sh->at("ff").num;
                         d.shared_limit = (float)sh->at("limit").num;
                     }
+                }
+                if (vov) {
+                    const Json& r = mlp->at("router");
+                    d.route_groups = d.route_keep = 1;
+                    d.route_scale = r.get("scale") ? (float)r.at("scale").num : 1.0f;
+                    if (const Json* gr = r.get("groups"))
+                        if (gr->truthy()) {
+                            d.route_groups = gr->get("count") ? (int)gr->at("count").num : 1;
+                            d.route_keep = gr->get("keep") ? (int)gr->at("keep").num : d.route_groups;
+                        }
+                    const Json* sh = mlp->get("shared");
+                    if (sh && sh->truthy()) d.shared_width = (int)sh->at("ff").num;
                 }
             } else {
                 throw std::runtime_error("config: unknown feed-forward kind '" + kind + "'");

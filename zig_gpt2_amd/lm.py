@@ -22,6 +22,14 @@ config.json (zig_gpt2_amd/models.py maps architecture names to loaders; `DESIGNS
   vectors added to the scaled embedding; experts with a clipped gated activation (`expert.limit`), chosen by their sigmoid
   scores, the score multiplying the expert's input; mlp.shared: an expert every token uses, times sigmoid(shared.sg . h);
   logit_scale, logit_softcap.
+  Vovalorn: type "gla" (gated linear attention: a decay per key channel, sigmoid(W_a2 W_a1 h + b)^(1 / tau); heads normed over
+  vdim, gated by silu(W_g h)) | "attention" (grouped-query attention over the whole sequence with no value projection —
+  a key head's un-normalised projection serves as its value —, q and k divided by their root mean square per head, a query factor that grows with the logarithm of the position
+  (q_temp: coef, every), scores capped (softcap) and lowered by a slope per head times the distance); a layer with "weights_of": j
+  runs layer j's tensors with separate cache and state; every norm is tanh(alpha v) * w + b (tensors `<name>`, `<name>.b`,
+  `<name>.alpha`), also behind the embedding (`embed.norm`); residual_mult: factor of every sublayer's normed output in the
+  residual sum; experts chosen by sigmoid scores + correction among the best contiguous blocks of experts (router.groups:
+  count, keep), weights normalised over the chosen, times router.scale; mlp.shared: an expert every token uses.
 """
 import ctypes as C
 import json
@@ -35,10 +43,12 @@ from . import _lib
 from ._lib import check_lm as check
 
 MIXERS = {"hgrn2": _lib.LM_MIX_HGRN2, "latent_attention": _lib.LM_MIX_LATENT_ATTENTION, "parallel": _lib.LM_MIX_PARALLEL,
-          "channel_delta": _lib.LM_MIX_CHANNEL_DELTA, "window_linear": _lib.LM_MIX_WINDOW_LINEAR}
+          "channel_delta": _lib.LM_MIX_CHANNEL_DELTA, "window_linear": _lib.LM_MIX_WINDOW_LINEAR, "gla": _lib.LM_MIX_GLA,
+          "attention": _lib.LM_MIX_ATTENTION}
 ROT_STYLES = {"yarn": _lib.LM_ROT_YARN, "bands": _lib.LM_ROT_BANDS}
 EXPERT_ACTS = {"glu_silu": _lib.LM_ACT_GLU_SILU, "gelu": _lib.LM_ACT_GELU, "glu_clipped": _lib.LM_ACT_GLU_CLIPPED}
-ROUTERS = {"softmax_all": _lib.LM_ROUTE_SOFTMAX_ALL, "top_logits": _lib.LM_ROUTE_TOP_LOGITS, "sigmoid_input": _lib.LM_ROUTE_SIGMOID_INPUT}
+ROUTERS = {"softmax_all": _lib.LM_ROUTE_SOFTMAX_ALL, "top_logits": _lib.LM_ROUTE_TOP_LOGITS, "sigmoid_input": _lib.LM_ROUTE_SIGMOID_INPUT,
+           "sigmoid_groups": _lib.LM_ROUTE_SIGMOID_GROUPS}
 
 # what an architecture name fixes beyond config.json.  mixers: layer type of config.json -> mixer of the library (two designs
 # call different pairs of branches "parallel")
@@ -49,6 +59,8 @@ DESIGNS = {
                     router="top_logits"),
     "Sanazen": dict(mixers={"parallel": "window_linear"}, tied_head=False, loop_readd=False, expert_act="glu_clipped", router="sigmoid_input",
                     side_by_side=True, sinusoid_positions=True),
+    "Vovalorn": dict(mixers={"gla": "gla", "attention": "attention"}, tied_head=False, loop_readd=False, expert_act="glu_silu", router="sigmoid_groups",
+                     tanh_norms=True, embed_norm=True),
 }
 
 
@@ -92,6 +104,15 @@ class LayerSpec:
     ff_limit: float = 0.0
     shared_width: int = 0
     shared_limit: float = 0.0
+    tau: float = 0.0  # gla: the decay is sigmoid(.)^(1 / tau)
+    softcap: float = 0.0  # attention: cap of the scores (0: none)
+    qtemp_coef: float = 0.0  # attention: the query factor 1 + coef ln(floor((p + 1) / every) + 1) ...
+    qtemp_every: int = 0  # ... 0: none
+    dist_bias: bool = False  # attention: head h loses 2^(-8 (h + 1) / heads) per position of distance
+    route_groups: int = 1  # sigmoid_groups: contiguous blocks of experts, how many of them stay in the race, factor of the weights
+    route_keep: int = 1
+    route_scale: float = 1.0
+    weights_of: Optional[int] = None  # this layer runs the tensors of that layer
 
     @classmethod
     def from_json(cls, entry, design="Tokosun", shapes=None, prefix=""):
@@ -102,7 +123,26 @@ class LayerSpec:
         if kind not in fixed["mixers"]:
             raise ValueError(f"unknown mixer type {kind!r} (known to {design}: {sorted(fixed['mixers'])})")
         kind = fixed["mixers"][kind]
-        if kind == "window_linear":
+
+        def inner(key, tensor):
+            """A size the configuration may leave to the checkpoint: rows of `tensor`."""
+            if key in m:
+                return int(m[key])
+            if shapes is None or prefix + tensor not in shapes:
+                raise KeyError(f"{prefix}mix: the inner size {key!r} needs the shape of tensor {prefix + tensor!r}")
+            return int(shapes[prefix + tensor][0])
+
+        if kind == "gla":
+            kw = dict(mixer=kind, heads=int(m["heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]), tau=float(m["tau"]),
+                      decay_rank=inner("decay_rank", "mix.a1"))
+        elif kind == "attention":
+            qt = m.get("q_temp") or {}
+            kw = dict(mixer=kind, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]),
+                      vdim=int(m.get("vdim", m["dim"])), scale=float(m["scale"]), softcap=float(m.get("softcap") or 0.0),
+                      qtemp_coef=float(qt.get("coef", 0.0)), qtemp_every=int(qt.get("every", 0)), dist_bias=bool(m.get("dist_bias", True)))
+            if kw["vdim"] != kw["dim"]:
+                raise ValueError(f"{prefix}mix: values reuse the key projection, so vdim {kw['vdim']} cannot differ from dim {kw['dim']}")
+        elif kind == "window_linear":
             l, r = m["left"], m["right"]
             mask = l.get("mask") or {}
             conv = l.get("conv")
@@ -122,13 +162,6 @@ class LayerSpec:
                       rot_base=float(rot.get("base", 10000.0)), rot_scaling=dict(rot["scaling"]) if rot.get("scaling") else None,
                       rot_style="bands", lru_width=int(r["width"]), lru_blocks=int(r["blocks"]), lru_conv=int(r["conv"]))
         elif kind == "channel_delta":
-            def inner(key, tensor):
-                if key in m:
-                    return int(m[key])
-                if shapes is None or prefix + tensor not in shapes:
-                    raise KeyError(f"{prefix}mix: the inner size {key!r} needs the shape of tensor {prefix + tensor!r}")
-                return int(shapes[prefix + tensor][0])
-
             kw = dict(mixer=kind, heads=int(m["heads"]), kv_heads=int(m.get("kv_heads", m["heads"])), dim=int(m["dim"]), vdim=int(m["vdim"]),
                       conv=int(m["conv"]), decay_rank=inner("decay_rank", "mix.a1"), gate_rank=inner("gate_rank", "mix.g1"))
         else:
@@ -149,8 +182,16 @@ class LayerSpec:
                     kw.update(ff_limit=float(mlp["expert"]["limit"]))
                     if mlp.get("shared"):
                         kw.update(shared_width=int(mlp["shared"]["ff"]), shared_limit=float(mlp["shared"]["limit"]))
+                elif mlp.get("shared"):
+                    kw.update(shared_width=int(mlp["shared"]["ff"]))
+                if fixed["router"] == "sigmoid_groups":
+                    groups = mlp["router"].get("groups") or {}
+                    count = int(groups.get("count", 1))
+                    kw.update(route_groups=count, route_keep=int(groups.get("keep", count)), route_scale=float(mlp["router"].get("scale", 1.0)))
             else:
                 raise ValueError(f"unknown feed-forward kind {mlp['kind']!r}")
+        if entry.get("weights_of") is not None:
+            kw.update(weights_of=int(entry["weights_of"]))
         return cls(**kw)
 
     def to_json(self):
@@ -176,6 +217,16 @@ class LayerSpec:
             if self.rot_scaling:
                 rot["scaling"] = dict(self.rot_scaling)
             mixer.update(rot_dim=self.rot_dim, kv_rank=self.kv_rank, q_rank=self.q_rank, scale=self.scale, rot=rot)
+        if self.mixer == "gla":
+            mixer.update(tau=self.tau, decay_rank=self.decay_rank)
+        elif self.mixer == "attention":
+            mixer.update(kv_heads=self.kv_heads, scale=self.scale)
+            if self.softcap:
+                mixer["softcap"] = self.softcap
+            if self.qtemp_every:
+                mixer["q_temp"] = {"coef": self.qtemp_coef, "every": self.qtemp_every}
+            if not self.dist_bias:
+                mixer["dist_bias"] = False
         mlp = None
         if self.ff == "dense":
             mlp = {"kind": "dense", "ff": self.ff_width}
@@ -184,7 +235,14 @@ class LayerSpec:
             if self.expert_act == "glu_clipped":
                 mlp["expert"]["limit"] = self.ff_limit
                 mlp["shared"] = {"ff": self.shared_width, "limit": self.shared_limit} if self.shared_width else None
-        return {"type": "parallel" if self.mixer == "window_linear" else self.mixer, "mixer": mixer, "mlp": mlp}
+            elif self.shared_width:
+                mlp["shared"] = {"ff": self.shared_width}
+            if self.router == "sigmoid_groups":
+                mlp["router"].update(groups={"count": self.route_groups, "keep": self.route_keep}, scale=self.route_scale)
+        out = {"type": "parallel" if self.mixer == "window_linear" else self.mixer, "mixer": mixer, "mlp": mlp}
+        if self.weights_of is not None:
+            out["weights_of"] = self.weights_of
+        return out
 
     def to_c(self):
         sc = self.rot_scaling or {}
@@ -196,14 +254,20 @@ class LayerSpec:
                             {"none": _lib.LM_FF_NONE, "dense": _lib.LM_FF_DENSE, "moe": _lib.LM_FF_MOE}[self.ff], self.ff_width, self.experts,
                             self.top, self.kv_heads, self.window, self.lru_width, self.lru_blocks, self.lru_conv, self.conv, self.decay_rank,
                             self.gate_rank, EXPERT_ACTS[self.expert_act], ROUTERS[self.router], self.keep_first, self.left_scale, self.right_scale,
-                            self.lin_heads, self.lin_dim, self.lin_vdim, self.ff_limit, self.shared_width, self.shared_limit)
+                            self.lin_heads, self.lin_dim, self.lin_vdim, self.ff_limit, self.shared_width, self.shared_limit, self.tau, self.softcap,
+                            self.qtemp_coef, self.qtemp_every, int(self.dist_bias), self.route_groups, self.route_keep, self.route_scale,
+                            0 if self.weights_of is None else self.weights_of + 1)
 
-    def tensor_shapes(self, prefix, width, canon_taps=0):
-        """{checkpoint tensor name: shape} of this layer."""
+    def tensor_shapes(self, prefix, width, canon_taps=0, tanh_norms=False):
+        """{checkpoint tensor name: shape} of this layer (none for a layer that runs another layer's tensors)."""
+        if self.weights_of is not None:
+            return {}
         H, D, V, W = self.heads, self.dim, self.vdim, width
         t = {prefix + "norm1": (W,), prefix + "norm1b": (W,)}
         if self.mixer == "window_linear":  # plain norms in front of the sublayers only, nothing between norm and mixer
             t = {prefix + "norm1": (W,)}
+        elif tanh_norms:  # the mixer reads the norm as it is
+            pass
         elif canon_taps:
             t[prefix + "canon1"] = (W, canon_taps)
             if self.ff != "none":
@@ -234,6 +298,12 @@ class LayerSpec:
                       m + "v": (H * V, W), m + "v.conv": (H * V, self.conv), m + "b": (H, W), m + "A_log": (H,), m + "norm": (V,),
                       m + "a1": (self.decay_rank, W), m + "a2": (H * D, self.decay_rank), m + "dt_bias": (H * D,),
                       m + "g1": (self.gate_rank, W), m + "g2": (H * V, self.gate_rank), m + "o": (W, H * V)})
+        elif self.mixer == "gla":
+            R = self.decay_rank
+            t.update({m + "q": (H * D, W), m + "k": (H * D, W), m + "v": (H * V, W), m + "g": (H * V, W), m + "o": (W, H * V), m + "norm": (V,),
+                      m + "a1": (R, W), m + "a2": (H * D, R), m + "a2.b": (H * D,)})
+        elif self.mixer == "attention":
+            t.update({m + "q": (H * D, W), m + "k": (self.kv_heads * D, W), m + "o": (W, H * D)})
         elif self.mixer == "hgrn2":
             t.update({m + "q": (H * D, W), m + "f": (H * D, W), m + "f.b": (H * D,), m + "lower": (H * D,), m + "v": (H * V, W), m + "norm": (V,),
                       m + "o": (W, H * V)})
@@ -258,7 +328,12 @@ class LayerSpec:
                 t[f + ("router.b" if self.router == "top_logits" else "correction")] = (self.experts,)
             if self.shared_width:
                 S = self.shared_width
-                t.update({f + "shared.gate": (S, W), f + "shared.up": (S, W), f + "shared.down": (W, S), f + "shared.sg": (1, W)})
+                t.update({f + "shared.gate": (S, W), f + "shared.up": (S, W), f + "shared.down": (W, S)})
+                if self.expert_act == "glu_clipped":
+                    t[f + "shared.sg"] = (1, W)
+        if tanh_norms:  # every norm's bias and scalar beside its weight
+            for name in [k for k in t if k[len(prefix):] in ("norm1", "norm1b", "norm2", "norm2b")]:
+                t.update({name + ".b": (W,), name + ".alpha": ()})
         return t
 
     def derived_tensors(self, prefix):
@@ -280,6 +355,7 @@ class LMConfig:
     canon_taps: int = 0  # > 0: both sublayers read h + conv(h) over this many tokens; 0: token shift in front of the mixer
     logit_scale: float = 1.0
     logit_softcap: float = 0.0  # > 0: logits <- cap tanh(logits / cap)
+    residual_mult: float = 1.0  # designs with tanh norms: factor of a sublayer's normed output in the residual sum
     extra: dict = field(default_factory=dict)
 
     @classmethod
@@ -288,11 +364,23 @@ class LMConfig:
         arch = cfg.get("architecture", "Tokosun")
         if arch not in DESIGNS:
             raise ValueError(f"architecture {arch!r} is not a layered design (known: {sorted(DESIGNS)})")
-        layers = [LayerSpec.from_json(e, arch, shapes, f"l{i}.") for i, e in enumerate(cfg["layers"])]
+        entries = cfg["layers"]
+
+        def owner(i):  # the layer whose tensors layer i runs
+            seen = set()
+            while entries[i].get("weights_of") is not None:
+                if i in seen or not 0 <= int(entries[i]["weights_of"]) < len(entries):
+                    raise ValueError(f"layer {i}: weights_of {entries[i]['weights_of']!r} names no layer with tensors")
+                seen.add(i)
+                i = int(entries[i]["weights_of"])
+            return i
+
+        layers = [LayerSpec.from_json(e, arch, shapes, f"l{owner(i)}.") for i, e in enumerate(entries)]
         return cls(vocab=int(cfg["vocab"]), width=int(cfg["width"]), layers=layers,
                    norm_eps=float(cfg["norm"]["eps"]), loop=dict(cfg["loop"]) if cfg.get("loop") else None, architecture=arch,
                    embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)), canon_taps=int((cfg.get("canon") or {}).get("taps", 0)),
-                   logit_scale=float(cfg.get("logit_scale") or 1.0), logit_softcap=float(cfg.get("logit_softcap") or 0.0))
+                   logit_scale=float(cfg.get("logit_scale") or 1.0), logit_softcap=float(cfg.get("logit_softcap") or 0.0),
+                   residual_mult=float(cfg.get("residual_mult", 1.0)))
 
     @classmethod
     def from_dir(cls, path):
@@ -315,6 +403,10 @@ class LMConfig:
             out["logit_scale"] = self.logit_scale
         if self.logit_softcap:
             out["logit_softcap"] = self.logit_softcap
+        if self.residual_mult != 1.0:
+            out["residual_mult"] = self.residual_mult
+        if out["loop"] is None and DESIGNS[self.architecture].get("tanh_norms"):
+            del out["loop"]
         return out
 
     @property
@@ -324,7 +416,8 @@ class LMConfig:
     def flags(self):
         d = DESIGNS[self.architecture]
         return ((_lib.LM_TIED_HEAD if d["tied_head"] else 0) | (_lib.LM_LOOP_READD if d["loop_readd"] else 0) |
-                (_lib.LM_SIDE_BY_SIDE if d.get("side_by_side") else 0) | (_lib.LM_SINUSOID_POSITIONS if d.get("sinusoid_positions") else 0))
+                (_lib.LM_SIDE_BY_SIDE if d.get("side_by_side") else 0) | (_lib.LM_SINUSOID_POSITIONS if d.get("sinusoid_positions") else 0) |
+                (_lib.LM_TANH_NORMS if d.get("tanh_norms") else 0) | (_lib.LM_EMBED_NORM if d.get("embed_norm") else 0))
 
     def passes(self):
         """Layer index of every pass, in execution order."""
@@ -336,10 +429,16 @@ class LMConfig:
 
     def tensor_shapes(self):
         t = {"embed": (self.vocab, self.width), "final.norm": (self.width,)}
+        d = DESIGNS[self.architecture]
+        tanh_norms = bool(d.get("tanh_norms"))
+        if tanh_norms:
+            t.update({"final.norm.b": (self.width,), "final.norm.alpha": ()})
+            if d.get("embed_norm"):
+                t.update({"embed.norm": (self.width,), "embed.norm.b": (self.width,), "embed.norm.alpha": ()})
         if not self.tied_head:
             t["head"] = (self.vocab, self.width)
         for i, l in enumerate(self.layers):
-            t.update(l.tensor_shapes(f"l{i}.", self.width, self.canon_taps))
+            t.update(l.tensor_shapes(f"l{i}.", self.width, self.canon_taps, tanh_norms))
         return t
 
     def derived_tensors(self):
@@ -364,7 +463,7 @@ class LayeredLM:
         cfg = _lib.LmConfig(config.vocab, config.width, len(config.layers), self._layers, int(loop["start"]), int(loop["stop"]), int(loop["times"]),
                             config.norm_eps, max_tokens, max_seqs, max_step_tokens, page_tokens,
                             (_lib.LM_F32 if dtype == "float32" else 0) | (0 if use_graph else _lib.LM_NO_GRAPH) | config.flags(),
-                            config.embed_scale, config.canon_taps, config.logit_scale, config.logit_softcap)
+                            config.embed_scale, config.canon_taps, config.logit_scale, config.logit_softcap, config.residual_mult)
         h = C.c_void_p()
         check(L.zg_lm_create(C.byref(h), C.byref(cfg), device))
         self.h = h
@@ -407,7 +506,8 @@ class LayeredLM:
                 if strict:
                     raise KeyError(f"tensor {name!r} is not part of this configuration")
                 continue
-            if tuple(np.shape(a)) != tuple(shapes[name]):
+            scalar = np.size(a) == 1 and int(np.prod(shapes[name], dtype=np.int64)) == 1  # a scalar may be stored as [] or [1]
+            if tuple(np.shape(a)) != tuple(shapes[name]) and not scalar:
                 raise ValueError(f"tensor {name!r} has shape {tuple(np.shape(a))}, the configuration needs {tuple(shapes[name])}")
             a = np.ascontiguousarray(a, dtype=np.float32)
             check(self._L.zg_lm_load_tensor(self.h, name.encode(), a.ctypes.data, a.size))

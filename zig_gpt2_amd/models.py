@@ -42,6 +42,13 @@ def _load_sanazen(path, dtype="bfloat16", **kw):
     return lm.LayeredLM.from_dir(path, dtype=dtype, **kw)
 
 
+@register("Vovalorn")
+def _load_vovalorn(path, dtype="bfloat16", **kw):
+    from . import lm
+
+    return lm.LayeredLM.from_dir(path, dtype=dtype, **kw)
+
+
 @register("gpt2")
 def _load_gpt2(path, dtype="float32", config="124M", **kw):
     from . import gpt

@@ -107,7 +107,7 @@ def read_safetensors(path):
 
 def bf16_bits_to_f32(bits):
     """uint16 bf16 bit patterns -> fp32 values (exact)."""
-    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+    return (np.ascontiguousarray(bits, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32).reshape(np.shape(bits))
 
 
 def load_safetensors_f32(path):
