@@ -48,9 +48,10 @@ def parse():
                    help="instead of the default workload: prompt and decode throughput of a layered model (Tokosun design, random weights) "
                         "at a size that resembles GPT-2 124M / medium / XL, beside the GPT-2 model of the same width and depth")
     p.add_argument("--lm-dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    p.add_argument("--lm-design", default="tokosun", choices=["tokosun", "gupizen", "sanazen"],
+    p.add_argument("--lm-design", default="tokosun", choices=["tokosun", "gupizen", "sanazen", "vovalorn"],
                    help="with --lm: which design is measured.  gupizen: a Gupizen stack of the same width and depth, beside the Tokosun stack "
-                        "(the tier's closest model) instead of GPT-2.  sanazen: a Sanazen stack beside the Gupizen stack of the same width and depth")
+                        "(the tier's closest model) instead of GPT-2.  sanazen: a Sanazen stack beside the Gupizen stack of the same width and depth.  "
+                        "vovalorn: a Vovalorn stack beside the Tokosun stack of the same width and depth")
     p.add_argument("--dry-run", action="store_true",
                    help="CPU rehearsal of the launch path (gloo, no GPU, no kernels): rendezvous, prompt sharding, "
                         "weight-arena broadcast, barriers and the max-reduce; prints a line with dry_run=true")
@@ -482,6 +483,27 @@ def sanazen_bench_config(width, n_layers, vocab, window=512):
                        embed_scale=1.0, logit_scale=1.0, logit_softcap=30.0)
 
 
+def vovalorn_bench_config(width, n_layers, vocab):
+    """A Vovalorn-design stack of `n_layers` layers in the repeating order gated linear attention, attention, attention, gated linear
+    attention (the order of the Tokosun stack beside it): recurrence heads of 128 x 128 (64 x 64 where the width does not divide)
+    with a decay projection of inner size 64, attention heads of 64 channels on a quarter as many key heads over the whole
+    context, every layer with 8 experts of width `width` in 2 groups of which one stays and 2 experts are chosen, and a shared
+    expert of the same width."""
+    from zig_gpt2_amd import lm
+
+    heads = width // 64
+    kv = heads // 4 if heads % 4 == 0 else heads // 5 if heads % 5 == 0 else heads
+    hd = 128 if width % 128 == 0 else 64
+    moe = dict(ff="moe", ff_width=width, experts=8, top=2, expert_act="glu_silu", router="sigmoid_groups", route_groups=2, route_keep=1,
+               route_scale=2.0, shared_width=width)
+    rec = dict(mixer="gla", heads=width // hd, dim=hd, vdim=hd, tau=8.0, decay_rank=64, **moe)
+    att = dict(mixer="attention", heads=heads, kv_heads=kv, dim=64, vdim=64, scale=64 ** -0.5, softcap=30.0, qtemp_coef=0.2, qtemp_every=128,
+               dist_bias=True, **moe)
+    order = [rec, att, att, rec]
+    return lm.LMConfig(vocab=vocab, width=width, layers=[lm.LayerSpec(**order[i % 4]) for i in range(n_layers)], norm_eps=1e-6,
+                       architecture="Vovalorn", residual_mult=0.5)
+
+
 def lm_weight_bytes(cfg):
     """(stored, read per decoded token) bytes of the bf16 matrices: every expert is stored, `top` of them are read."""
     stored = active = 0
@@ -508,6 +530,7 @@ def lm_bench(a):
     ctx = a.ctx or 1024
     gup = a.lm_design == "gupizen"
     san = a.lm_design == "sanazen"
+    vov = a.lm_design == "vovalorn"
     cfg = lm_bench_config(width, n_layers, gcfg.vocab_size)
     out = {"metric": "lm_decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if a.lm_dtype == "bfloat16" else "fp32", "data": "synthetic (random weights, filled on the GPU)",
@@ -567,6 +590,15 @@ def lm_bench(a):
         out["config"]["model"] = (f"Sanazen design, width {width}, {n_layers} layers (window 512 + 4 kept tokens beside linear attention; 8 experts, "
                                   f"2 chosen, one shared), vocab {gcfg.vocab_size}")
         out.update(value=d1["tokens_per_s"], ms_per_step=round(d1["wall_us_per_step"] / 1e3, 4), sanazen=s_res, gupizen_equal_size=g_res)
+        print(json.dumps(out))
+        return
+    if vov:  # beside the tier's closest model (a recurrence with a decay per key channel, attention over the whole context, gated experts)
+        v_res = measure(vovalorn_bench_config(width, n_layers, gcfg.vocab_size))
+        t_res = measure(lm_bench_config(width, n_layers, gcfg.vocab_size))
+        d1 = v_res["decode"][0]
+        out["config"]["model"] = (f"Vovalorn design, width {width}, {n_layers} layers (gated linear attention, attention x2, gated linear attention; "
+                                  f"8 experts in 2 groups, 2 chosen, one shared), vocab {gcfg.vocab_size}")
+        out.update(value=d1["tokens_per_s"], ms_per_step=round(d1["wall_us_per_step"] / 1e3, 4), vovalorn=v_res, tokosun_equal_size=t_res)
         print(json.dumps(out))
         return
     if gup:  # the new design beside the tier's closest model at equal width and depth
