@@ -374,6 +374,25 @@ def test_long_decoding(dtype):
     m.close()
 
 
+def test_decoding_across_length_buckets():
+    """Decode steps replay a graph per bucket of the longest sequence's length (512, 1024, ... tokens: a row's keys are split into
+    shares by the bucket's capacity).  Two sequences decode in lock step while the longer one crosses 512 and 1024."""
+    cfg = vl.config([vl.attn_layer(heads=4, kv_heads=2, dim=8, q_temp=(0.5, 100)), vl.gla_layer(heads=1, dim=8, vdim=8)], width=24, vocab=61)
+    w = vl.weights(cfg, seed=31)
+    a, b = vl.tokens(65, 1040, cfg["vocab"]), vl.tokens(66, 560, cfg["vocab"])
+    ra, rb = vo.forward(w, cfg, a), vo.forward(w, cfg, b)
+    m = make(cfg, w, max_tokens=2048)
+    sa, sb = m.open(), m.open()
+    m.step([(sa, a[:505], []), (sb, b[:25], [])])
+    for lo, n in ((505, 15), (1015, 25)):  # 505 .. 519 and 1015 .. 1039 of the longer sequence
+        if lo == 1015:
+            m.step([(sa, a[520:1015], []), (sb, b[40:535], [])])
+        rows = [m.step([(sa, a[lo + t:lo + t + 1], [0]), (sb, b[lo - 480 + t:lo - 479 + t], [0])]) for t in range(n)]
+        tl.assert_close(np.stack([r[0] for r in rows]), ra[lo:lo + n], "float32", lo)
+        tl.assert_close(np.stack([r[1] for r in rows]), rb[lo - 480:lo - 480 + n], "float32", lo)
+    m.close()
+
+
 def test_decode_steps_with_and_without_the_captured_graph():
     """A decode step replays the graph captured for its batch size; every replay, with eager prompt steps of other sequences
     between them, equals the same step launched kernel by kernel."""

@@ -224,7 +224,12 @@ struct zg_lm {
     float last_step_ms = 0.0f, last_decode_ms = 0.0f;
     bool use_graph = true;
     int step_keys = 0;  // positions the longest sequence of the running portion has reached (what its rows can see at most)
-    hipGraphExec_t decode_graph[kGemvMaxRows + 1] = {};  // by rows of the step (one per entry)
+    // by rows of the step (one per entry) and, where whole-context attention splits a row's keys into shares, by the length bucket
+    // of the longest sequence (512, 1024, ... tokens): a share then holds a few dozen keys at any length
+    static constexpr int kKeyBuckets = 24;
+    hipGraphExec_t decode_graph[kGemvMaxRows + 1][kKeyBuckets] = {};
+    bool whole_context = false;  // some pass attends over the whole sequence through the split kernels
+    int bucket_keys = 0;         // key capacity of the running decode step's bucket
 };
 
 namespace {
@@ -950,7 +955,7 @@ int enqueue_layers(zg_lm* g, int M, int n_ent, bool capturing, bool single) {
             // rows of the score workspace: as long as the longest sequence of this portion (a captured decode step replays at any
             // length, so it takes the cache's capacity)
             const int all_keys = g->max_pages * g->P;
-            const int key_cap = (single || capturing) ? all_keys : std::min(all_keys, (g->step_keys + 63) / 64 * 64);
+            const int key_cap = (single || capturing) ? (g->bucket_keys > 0 ? g->bucket_keys : all_keys) : std::min(all_keys, (g->step_keys + 63) / 64 * 64);
             bool split = false;
             ZG_TRY(launch_window_attention_split(g->proj, NP, g->o, HD, M, H, G, D, D, d.scale, 0, 0, nullptr, nullptr, nullptr, d_pos, d_slot,
                                                  g->page_table, g->max_pages, g->P, ps.cache, key_cap, g->win_ws, g->win_ws_floats, d_estart, d_elen,
@@ -1275,8 +1280,15 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
     ZG_HIP(hipEventRecord(g->ev0, s));
     bool single = M <= kGemvMaxRows && !g->trace && g->use_graph;
     for (const Piece& pc : pieces) single = single && pc.n == 1;
+    int bucket = 0;
+    g->bucket_keys = 0;
+    if (g->whole_context) {  // the smallest bucket that holds the longest sequence of the step
+        const int all_keys = g->max_pages * g->P;
+        while (bucket + 1 < zg_lm::kKeyBuckets && (512LL << bucket) < g->step_keys) ++bucket;
+        g->bucket_keys = (int)std::min<long long>(all_keys, 512LL << bucket);
+    }
     if (single) {  // a decode step: replay the captured sequence of this batch size
-        if (!g->decode_graph[M]) {
+        if (!g->decode_graph[M][bucket]) {
             hipGraph_t graph = nullptr;
             ZG_HIP(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
             const int st = enqueue_layers(g, M, n_ent, true, true);
@@ -1286,10 +1298,10 @@ int run_portion(zg_lm* g, const std::vector<Piece>& pieces, float* logits_out, c
                 return st;
             }
             ZG_HIP(ce);
-            ZG_HIP(hipGraphInstantiate(&g->decode_graph[M], graph, nullptr, nullptr, 0));
+            ZG_HIP(hipGraphInstantiate(&g->decode_graph[M][bucket], graph, nullptr, nullptr, 0));
             ZG_HIP(hipGraphDestroy(graph));
         }
-        ZG_HIP(hipGraphLaunch(g->decode_graph[M], s));
+        ZG_HIP(hipGraphLaunch(g->decode_graph[M][bucket], s));
     } else {
         bool one_row = M <= kGemvMaxRows;
         for (const Piece& pc : pieces) one_row = one_row && pc.n == 1;
@@ -1547,6 +1559,7 @@ int zg_lm_create(zg_lm** out, const zg_lm_config* config, int device) {
         const zg_lm_layer& d = g->layers[ps.layer].d;
         if (d.mixer == ZG_LM_MIX_LATENT_ATTENTION || d.mixer == ZG_LM_MIX_ATTENTION || (d.mixer == ZG_LM_MIX_PARALLEL && d.window == 0))
             attends = true, bounded = false;
+        if (d.mixer == ZG_LM_MIX_ATTENTION) g->whole_context = true;
         if (d.mixer == ZG_LM_MIX_PARALLEL && d.window > 0) {
             attends = true;
             g->keep_tokens = std::max(g->keep_tokens, d.window);
@@ -1643,8 +1656,9 @@ int zg_lm_destroy(zg_lm* g) {
     if (!g) return ZG_OK;
     (void)hipSetDevice(g->device);
     if (g->stream) (void)hipStreamSynchronize(g->stream);
-    for (hipGraphExec_t e : g->decode_graph)
-        if (e) (void)hipGraphExecDestroy(e);
+    for (auto& by_rows : g->decode_graph)
+        for (hipGraphExec_t e : by_rows)
+            if (e) (void)hipGraphExecDestroy(e);
     if (g->ev0) (void)hipEventDestroy(g->ev0);
     if (g->ev1) (void)hipEventDestroy(g->ev1);
     if (g->stream) (void)hipStreamDestroy(g->stream);

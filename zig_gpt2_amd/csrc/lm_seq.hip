@@ -697,7 +697,10 @@ __global__ __launch_bounds__(256) void window_mix_kernel(int H, int G, int D, in
 // the block's key range go to blockIdx.y (the merge adds them), groups of kPvUnits * 4 units to blockIdx.z.
 constexpr int kPvKeys = 16;
 constexpr int kPvUnits = 3;  // (head, channel tile) units a wave accumulates (few: two workgroups share a compute unit and hide each other's loads)
-constexpr int kPvHeads = 16; // most heads of this form (a pair's weights of all heads sit in registers)
+constexpr int kPvHeads = 16; // most heads a workgroup weighs (a pair's weights of these heads sit in registers)
+// Without a mixing matrix the heads are independent: a workgroup then weighs only the heads of its own units (at most
+// pv_block_heads of them), so any number of heads fits and no score is read by more than one group of units.
+__host__ __device__ constexpr int pv_block_heads(int ctiles) { return (4 * kPvUnits - 1) / ctiles + 2; }
 
 __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int D, int V, int window, int keep, const float* sink, const float* talk,
                                                               const int* ent_start, const int* ent_len, int n_entries, const int* row_pos,
@@ -706,8 +709,14 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
                                                               float* po) {
     extern __shared__ __attribute__((aligned(16))) float s_pv[];
     constexpr int KP = kPvKeys + 1;           // padded key stride
-    float* s_w = s_pv;                        // [H][32][KP] mixed weights of the tile
-    float* s_talk = s_w + H * 32 * KP;        // [H H]
+    const int ctiles = (V + 31) / 32, units = H * ctiles;
+    // the heads this workgroup weighs: all of them under a mixing matrix, else those of its own units
+    const int ub0 = blockIdx.z * 4 * kPvUnits;
+    const int h_lo = talk ? 0 : min(H - 1, ub0 / ctiles);
+    const int h_n = talk ? H : min(H, (ub0 + 4 * kPvUnits - 1) / ctiles + 1) - h_lo;
+    const int hs = talk ? H : min(H, pv_block_heads(ctiles));
+    float* s_w = s_pv;                        // [hs][32][KP] mixed weights of the tile (head h at h - h_lo)
+    float* s_talk = s_w + hs * 32 * KP;       // [H H]
     float* s_M = s_talk + H * H;              // [32][H]
     float* s_iZ = s_M + 32 * H;               // [32][H]
     __shared__ int s_row[kPvKeys];
@@ -721,9 +730,10 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
     const int n_tiles = (n_blk - 1) / kPvKeys + 1, per = (n_tiles + gridDim.y - 1) / gridDim.y;
     const int t_lo = min(n_tiles, (int)blockIdx.y * per), t_hi = min(n_tiles, t_lo + per);
     const int* pages = page_table + (size_t)row_slot[m0] * max_pages;
-    const int rep = H / G, ctiles = (V + 31) / 32, units = H * ctiles;
+    const int rep = H / G;
     const size_t cstride = (size_t)G * (D + V);
-    for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk ? talk[i] : ((i / H) == (i % H) ? 1.0f : 0.0f);
+    if (talk)
+        for (int i = tid; i < H * H; i += blockDim.x) s_talk[i] = talk[i];
     for (int i = tid; i < 32 * H; i += blockDim.x) {  // the rows' maximum and denominator per head, the sink counted once
         const int row = i / H, h = i % H;
         float mx = 0.0f, iz = 0.0f;
@@ -755,13 +765,14 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
             const KeySpan sp = key_span(pi, window, keep);
             const bool ok = row < nrows && j <= pi && (j >= sp.j_lo || j < sp.n_first);
             float p[kPvHeads];  // (registers: the loops over it are unrolled to the kernel's most heads)
-            const float* sr = sc + (size_t)(m0 + min(row, nrows - 1)) * H * NK + (ok ? (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j) : 0);
+            const float* sr = sc + ((size_t)(m0 + min(row, nrows - 1)) * H + h_lo) * NK + (ok ? (j >= sp.j_lo ? sp.n_first + (j - sp.j_lo) : j) : 0);
 #pragma unroll
-            for (int g = 0; g < kPvHeads; ++g) p[g] = (ok && g < H) ? expf(sr[(size_t)g * NK] - s_M[row * H + g]) * s_iZ[row * H + g] : 0.0f;
+            for (int g = 0; g < kPvHeads; ++g)
+                p[g] = (ok && g < h_n) ? expf(sr[(size_t)g * NK] - s_M[row * H + h_lo + g]) * s_iZ[row * H + h_lo + g] : 0.0f;
             if (!talk) {  // no mixing matrix: every head keeps its own weights
 #pragma unroll
                 for (int g = 0; g < kPvHeads; ++g)
-                    if (g < H) s_w[(g * 32 + row) * KP + kk] = p[g];
+                    if (g < h_n) s_w[(g * 32 + row) * KP + kk] = p[g];
                 continue;
             }
             for (int h = 0; h < H; ++h) {
@@ -784,7 +795,7 @@ __global__ __launch_bounds__(256) void window_mix_mfma_kernel(int H, int G, int 
         for (int u = 0; u < kPvUnits; ++u) {
             const int unit = u0 + u;
             if (unit < units) {
-                const float* wrow = s_w + ((unit / ctiles) * 32 + r) * KP + kh * (kPvKeys / 2);
+                const float* wrow = s_w + ((unit / ctiles - h_lo) * 32 + r) * KP + kh * (kPvKeys / 2);
 #pragma unroll
                 for (int t = 0; t < kPvKeys / 2; ++t) acc[u] = __builtin_amdgcn_mfma_f32_32x32x2f32(wrow[t], vv[u][t], acc[u], 0, 0, 0);
             }
@@ -1372,8 +1383,10 @@ int launch_window_attention_split(const float* q, int ldq, float* out, int ldo, 
 #undef ZG_WS
         ZG_HIP(hipGetLastError());
     }
-    const size_t lds_c = ((size_t)H * 32 * (kPvKeys + 1) + (size_t)H * H + 64 * (size_t)H) * sizeof(float);
-    if (tiled && H <= kPvHeads && lds_c <= 60 * 1024) {  // the value product of 32 rows at a time on the matrix cores
+    const bool mixes = talk != nullptr;  // (a mixing matrix: a workgroup weighs every head, else only those of its units)
+    const int hs = mixes ? H : std::min(H, pv_block_heads((V + 31) / 32));
+    const size_t lds_c = ((size_t)hs * 32 * (kPvKeys + 1) + (size_t)H * H + 64 * (size_t)H) * sizeof(float);
+    if (tiled && (!mixes || H <= kPvHeads) && lds_c <= 60 * 1024) {  // the value product of 32 rows at a time on the matrix cores
         const int units = H * ((V + 31) / 32);
         const dim3 pg((M + 31) / 32 + n_entries, n_split, (units + 4 * kPvUnits - 1) / (4 * kPvUnits));
         window_mix_mfma_kernel<<<pg, 256, lds_c, s>>>(H, G, D, V, window, keep, sink, talk, ent_start, ent_len, n_entries, row_pos, row_slot, page_table,
